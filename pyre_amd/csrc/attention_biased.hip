@@ -11,7 +11,9 @@
 //   out_i = gate_i * out_scale * sum_j softmax_j(s(i, .)) v_j
 //
 // `bias` is the table by distance that the host made of the model's buckets: [nq][far + 1] float32,
-// or null. `gate` is float32 [n][nq] (already squashed), or null.
+// or null. `gate` is float32 [n][nq] (already squashed; gate_dim = 1) or [n][nq * dv] (a gate per element of the
+// output; gate_dim = dv), or null. `sink` is float32 [nq] or null: exp(sink[head]) joins the softmax's denominator,
+// a key that has no value (it is neither scaled nor capped nor biased).
 //
 // unit_qkv_write  finishes the input product of a step (partial sums), divides every query and key
 //                 head by its root mean square, stores queries, keys and values and the squashed gates.
@@ -157,6 +159,15 @@ __device__ inline int first_seen(int pos, int window, int chunk) {
   return lo;
 }
 
+// The softmax's last factor with a sink in the denominator: the output sums were made against the maximum m and the
+// sum l; with M = max(m, sink) they are worth e^(m - M) / (l e^(m - M) + e^(sink - M)).
+__device__ inline float softmax_factor(float m, float l, const float* sink, int head) {
+  if (!sink) return l > 0.f ? 1.f / l : 0.f;
+  const float sk = sink[head], M = fmaxf(m, sk);
+  const float a = m == -INFINITY ? 0.f : expf(m - M);
+  return a / (l * a + expf(sk - M));
+}
+
 __device__ inline float shaped_score(float raw, float scale, float cap, const float* bias_row, int dist, int far) {
   float s = raw * scale;
   if (cap > 0.f) s = cap * tanh_by_exp(s / cap);
@@ -176,7 +187,8 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
     int out_ld, const float* __restrict__ gate, float out_scale, const int* __restrict__ tiles,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, int nq, int nkv, int dk, int dkp, int dv, int page_size, float scale, float cap,
-    const float* __restrict__ bias, int far, int window, int keep_first, int chunk, int tab_lds, int bias_lds) {
+    const float* __restrict__ bias, int far, int window, int keep_first, int chunk, int tab_lds, int bias_lds,
+    const float* __restrict__ sink, int gate_dim) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   // rows of keys and queries hold the even elements first, then the odd ones: a lane's operands of four
   // steps of the first product are then one 16-byte read
@@ -373,15 +385,16 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
   if (!active) return;
   l += __shfl_xor(l, 32, 64);
   if (!live) return;
-  float f = (l > 0.f ? 1.f / l : 0.f) * out_scale;
-  if (gate) f *= gate[static_cast<size_t>(t0 + c) * nq + head];
+  float f = softmax_factor(m, l, sink, head) * out_scale;
+  const float* grow = gate ? gate + (static_cast<size_t>(t0 + c) * nq + head) * gate_dim : nullptr;
+  if (gate && gate_dim == 1) f *= grow[0];
   T* dst = out + static_cast<size_t>(t0 + c) * out_ld + head * dv;
 #pragma unroll
   for (int dt = 0; dt < NV; ++dt)
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int d = 32 * dt + 8 * (i >> 2) + 4 * h + (i & 3);
-      if (d < dv) dst[d] = from_float<T>(o[dt][i] * f);
+      if (d < dv) dst[d] = from_float<T>(o[dt][i] * (gate_dim > 1 && gate ? f * grow[d] : f));
     }
 }
 
@@ -405,7 +418,8 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile16_kernel(
     int out_ld, const float* __restrict__ gate, float out_scale, const int* __restrict__ tiles,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, int nq, int nkv, int dk, int dkp, int dv, int page_size, float scale, float cap,
-    const float* __restrict__ bias, int far, int window, int keep_first, int chunk, int tab_lds, int bias_lds) {
+    const float* __restrict__ bias, int far, int window, int keep_first, int chunk, int tab_lds, int bias_lds,
+    const float* __restrict__ sink, int gate_dim) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   const int ldk = dkp + kPad16, ldv = kKeys + kPad16;
   bf16* Ks = reinterpret_cast<bf16*>(lds_raw);                 // [kKeys][ldk]
@@ -591,15 +605,16 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile16_kernel(
   if (!active) return;
   l += __shfl_xor(l, 32, 64);
   if (!live) return;
-  float f = (l > 0.f ? 1.f / l : 0.f) * out_scale;
-  if (gate) f *= gate[static_cast<size_t>(t0 + c) * nq + head];
+  float f = softmax_factor(m, l, sink, head) * out_scale;
+  const float* grow = gate ? gate + (static_cast<size_t>(t0 + c) * nq + head) * gate_dim : nullptr;
+  if (gate && gate_dim == 1) f *= grow[0];
   bf16* dst = out + static_cast<size_t>(t0 + c) * out_ld + head * dv;
 #pragma unroll
   for (int dt = 0; dt < NV; ++dt)
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int d = 32 * dt + 8 * (i >> 2) + 4 * h + (i & 3);
-      if (d < dv) dst[d] = from_float<bf16>(o[dt][i] * f);
+      if (d < dv) dst[d] = from_float<bf16>(o[dt][i] * (gate_dim > 1 && gate ? f * grow[d] : f));
     }
 }
 
@@ -618,7 +633,8 @@ __global__ __launch_bounds__(kThreads) void attn_biased_single_kernel(
     int out_ld, const float* __restrict__ gate, float out_scale, const int* __restrict__ tokens,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale, float cap,
-    const float* __restrict__ bias, int far, int window, int keep_first, int chunk, int hg, float* __restrict__ part) {
+    const float* __restrict__ bias, int far, int window, int keep_first, int chunk, int hg, float* __restrict__ part,
+    const float* __restrict__ sink, int gate_dim) {
   __shared__ __attribute__((aligned(16))) float qs[kGroup][kMaxHead];
   __shared__ float sc[kGroup][kSpan];
   __shared__ int row_s[kSpan];
@@ -736,9 +752,8 @@ __global__ __launch_bounds__(kThreads) void attn_biased_single_kernel(
       if (dd == 0) dst[dv] = m_s[a], dst[dv + 1] = l_s[a];
       continue;
     }
-    const float l = l_s[a];
-    float f = (l > 0.f ? 1.f / l : 0.f) * out_scale;
-    if (gate) f *= gate[static_cast<size_t>(n) * nq + h];
+    float f = softmax_factor(m_s[a], l_s[a], sink, h) * out_scale;
+    if (gate) f *= gate[(static_cast<size_t>(n) * nq + h) * gate_dim + (gate_dim > 1 ? dd : 0)];
     out[static_cast<size_t>(n) * out_ld + h * dv + dd] = from_float<T>(total * f);
   }
 }
@@ -748,7 +763,7 @@ template <typename T>
 __global__ __launch_bounds__(kThreads) void attn_biased_join_kernel(
     const float* __restrict__ part, T* __restrict__ out, int out_ld, const float* __restrict__ gate, float out_scale,
     const int* __restrict__ tokens, const int* __restrict__ positions, int nq, int dv, int window, int keep_first,
-    int chunk, int max_spans) {
+    int chunk, int max_spans, const float* __restrict__ sink, int gate_dim) {
   const int n = tokens ? tokens[blockIdx.x] : blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int pos = positions[n];
   const int lo = first_seen(pos, window, chunk);
@@ -757,6 +772,7 @@ __global__ __launch_bounds__(kThreads) void attn_biased_join_kernel(
   const float* src = part + (static_cast<size_t>(blockIdx.x) * nq + h) * max_spans * (dv + 2);
   float M = -INFINITY;
   for (int s = 0; s < spans; ++s) M = fmaxf(M, src[s * (dv + 2) + dv]);
+  if (sink) M = fmaxf(M, sink[h]);
   const float m_use = M == -INFINITY ? 0.f : M;
   if (tid < dv) {
     float total = 0.f, l = 0.f;
@@ -765,8 +781,9 @@ __global__ __launch_bounds__(kThreads) void attn_biased_join_kernel(
       total = fmaf(src[s * (dv + 2) + tid], w, total);
       l = fmaf(src[s * (dv + 2) + dv + 1], w, l);
     }
+    if (sink) l += expf(sink[h] - m_use);
     float f = (l > 0.f ? 1.f / l : 0.f) * out_scale;
-    if (gate) f *= gate[static_cast<size_t>(n) * nq + h];
+    if (gate) f *= gate[(static_cast<size_t>(n) * nq + h) * gate_dim + (gate_dim > 1 ? tid : 0)];
     out[static_cast<size_t>(n) * out_ld + h * dv + tid] = from_float<T>(total * f);
   }
 }
@@ -812,8 +829,9 @@ extern "C" int pyre_attn_biased_tile(const void* q, void* out, int out_ld, int d
                                      const int* positions, const int* seq_of_token, const int* block_table,
                                      int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale,
                                      float cap, const float* bias, int far, int window, int keep_first, int chunk,
-                                     hipStream_t stream) {
+                                     const float* sink, int gate_dim, hipStream_t stream) {
   if (check_geometry("attn_biased_tile", nq, nkv, dk, dv, page_size)) return 1;
+  PYRE_REQUIRE(gate_dim == 1 || gate_dim == dv, "attn_biased_tile: a gate per head or per element, not per %d", gate_dim);
   PYRE_REQUIRE(known_dtype(dt) && table_stride > 0 && window >= 0 && keep_first >= 0 && far >= 0 && chunk >= 0, "attn_biased_tile: bad arguments");
   PYRE_REQUIRE(dk <= kTileMaxKeyHead, "attn_biased_tile: key heads of %d elements are more than %d", dk, kTileMaxKeyHead);
   if (n_tiles <= 0) return 0;
@@ -841,7 +859,7 @@ extern "C" int pyre_attn_biased_tile(const void* q, void* out, int out_ld, int d
     hipLaunchKernelGGL((attn_biased_tile_kernel<T, NV, VEC>), grid, dim3(kThreads), lds, stream, static_cast<const T*>(q), \
                        static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), static_cast<T*>(out), out_ld, \
                        gate, out_scale, tiles, positions, seq_of_token, block_table, table_stride, nq, nkv, dk, dkp,  \
-                       dv, page_size, scale, cap, bias, far, window, keep_first, chunk, tab_lds, bias_lds);                 \
+                       dv, page_size, scale, cap, bias, far, window, keep_first, chunk, tab_lds, bias_lds, sink, gate_dim); \
   } while (0)
 #define PYRE_TILE_NV(T, VEC)                \
   switch (nvp) {                            \
@@ -872,7 +890,8 @@ extern "C" int pyre_attn_biased_tile(const void* q, void* out, int out_ld, int d
     hipLaunchKernelGGL((attn_biased_tile16_kernel<NV>), grid, dim3(kThreads), lds16, stream, static_cast<const bf16*>(q), \
                        static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), static_cast<bf16*>(out),    \
                        out_ld, gate, out_scale, tiles, positions, seq_of_token, block_table, table_stride, nq, nkv, dk,  \
-                       dkp, dv, page_size, scale, cap, bias, far, window, keep_first, chunk, tab16, bias16);             \
+                       dkp, dv, page_size, scale, cap, bias, far, window, keep_first, chunk, tab16, bias16, sink,         \
+                       gate_dim);                                                                                        \
   } while (0)
     switch (nvp) {
       case 1: PYRE_TILE16(1); break;
@@ -906,8 +925,10 @@ extern "C" int pyre_attn_biased_single(const void* q, void* out, int out_ld, int
                                        int n, const int* positions, const int* seq_of_token, const int* block_table,
                                        int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale,
                                        float cap, const float* bias, int far, int window, int keep_first, int chunk,
-                                       float* part, int max_spans, hipStream_t stream) {
+                                       float* part, int max_spans, const float* sink, int gate_dim,
+                                       hipStream_t stream) {
   if (check_geometry("attn_biased_single", nq, nkv, dk, dv, page_size)) return 1;
+  PYRE_REQUIRE(gate_dim == 1 || gate_dim == dv, "attn_biased_single: a gate per head or per element, not per %d", gate_dim);
   PYRE_REQUIRE(known_dtype(dt) && table_stride > 0 && window >= 0 && keep_first >= 0 && far >= 0 && chunk >= 0, "attn_biased_single: bad arguments");
   PYRE_REQUIRE(!part || (max_spans >= 1 && max_spans <= 65535), "attn_biased_single: %d spans are not a launch", max_spans);
   if (n <= 0) return 0;
@@ -931,7 +952,8 @@ extern "C" int pyre_attn_biased_single(const void* q, void* out, int out_ld, int
       hipLaunchKernelGGL((attn_biased_single_kernel<T, VEC>), grid, dim3(kThreads), 0, stream,                            \
                          static_cast<const T*>(q), static_cast<const T*>(k_cache), static_cast<const T*>(v_cache),        \
                          static_cast<T*>(out), out_ld, gate, out_scale, tokens, positions, seq_of_token, block_table,     \
-                         table_stride, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first, chunk, hg, part))
+                         table_stride, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first, chunk, hg, part, \
+                         sink, gate_dim))
   if (dk % 8 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0) {
     PYRE_SINGLE(true);
   } else {
@@ -941,6 +963,7 @@ extern "C" int pyre_attn_biased_single(const void* q, void* out, int out_ld, int
   if (part)
     PYRE_DISPATCH(dt, T,
         hipLaunchKernelGGL(attn_biased_join_kernel<T>, dim3(n, nq), dim3(kThreads), 0, stream, part, static_cast<T*>(out),
-                           out_ld, gate, out_scale, tokens, positions, nq, dv, window, keep_first, chunk, max_spans));
+                           out_ld, gate, out_scale, tokens, positions, nq, dv, window, keep_first, chunk, max_spans, sink,
+                           gate_dim));
   return check_launch("attn_biased_single");
 }

@@ -30,6 +30,48 @@ extern "C" int pyre_embed(const void* table, int table_dt, const int* ids, float
   return check_launch("embed");
 }
 
+// out[n] = table[ids[n]] + pairs[row]: row = (previous token * mul_prev + ids[n] * mul_cur) mod buckets, or `buckets`
+// (the table's last row) for a request's first token. The token before the first one that a request brings in this step
+// is what the request's state holds (a float32 whose value is the token's number); the block of that first token reads
+// it and then leaves the request's last token of the step there, so no other block touches the state.
+template <typename T>
+__global__ void bigram_embed_kernel(const T* __restrict__ table, const T* __restrict__ pairs, const int* __restrict__ ids,
+                                    const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+                                    const int* __restrict__ q_start, float* __restrict__ state,
+                                    const int* __restrict__ state_slots, float* __restrict__ out, int hidden, int buckets,
+                                    int mul_prev, int mul_cur) {
+  __shared__ int row_s;
+  const int n = blockIdx.x;
+  if (threadIdx.x == 0) {
+    const int s = seq_of_token[n], first = q_start[s], tok = ids[n];
+    long long prev = 0;
+    if (n > first) prev = ids[n - 1];
+    else if (positions[n] > 0) prev = static_cast<long long>(state[state_slots[s]]);
+    row_s = positions[n] == 0 ? buckets
+                              : static_cast<int>((prev * mul_prev + static_cast<long long>(tok) * mul_cur) % buckets);
+    if (n == first) state[state_slots[s]] = static_cast<float>(ids[q_start[s + 1] - 1]);
+  }
+  __syncthreads();
+  const T* row = table + static_cast<size_t>(ids[n]) * hidden;
+  const T* pair = pairs + static_cast<size_t>(row_s) * hidden;
+  float* o = out + static_cast<size_t>(n) * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = to_float(row[i]) + to_float(pair[i]);
+}
+
+extern "C" int pyre_bigram_embed(const void* table, const void* pairs, int dt, const int* ids, const int* positions,
+                                 const int* seq_of_token, const int* q_start, float* state, const int* state_slots,
+                                 float* out, int n, int hidden, int buckets, int mul_prev, int mul_cur, hipStream_t stream) {
+  PYRE_REQUIRE(known_dtype(dt), "bigram_embed: unknown table dtype %d", dt);
+  PYRE_REQUIRE(n >= 0 && hidden > 0 && buckets > 0 && mul_prev >= 0 && mul_cur >= 0, "bigram_embed: bad sizes");
+  PYRE_REQUIRE(state && state_slots && q_start && seq_of_token && positions, "bigram_embed: the step's arrays and the state are needed");
+  if (n == 0) return 0;
+  PYRE_DISPATCH(dt, T,
+                hipLaunchKernelGGL(bigram_embed_kernel<T>, dim3(n), dim3(256), 0, stream, static_cast<const T*>(table),
+                                   static_cast<const T*>(pairs), ids, positions, seq_of_token, q_start, state, state_slots,
+                                   out, hidden, buckets, mul_prev, mul_cur));
+  return check_launch("bigram_embed");
+}
+
 // ---------------------------------------------------------------------------
 // resid += sum_p delta[p] (+ bias);  out = resid * rsqrt(mean(resid^2) + eps) * gain
 // (pyre/model.py:33-38 for the norm, :151-152 for the residual sums).

@@ -90,7 +90,7 @@ __global__ __launch_bounds__(kThreads) void gla_prepare_vec_kernel(
 template <int DR>
 __global__ __launch_bounds__(kThreads) void gla_scan_kernel(
     const float* __restrict__ x, float* __restrict__ state, float* __restrict__ o, const int* __restrict__ q_start,
-    const int* __restrict__ state_slots, int heads, int dk, int dv, float qscale) {
+    const int* __restrict__ state_slots, int heads, int dk, int dv, float qscale, const float* __restrict__ decay) {
   __shared__ float red[2][4][kWave];
   const int s = blockIdx.x, hd = blockIdx.y, tid = threadIdx.x, w = tid >> 6, lane = tid & 63;
   const int col = blockIdx.z * kWave + lane;
@@ -104,6 +104,7 @@ __global__ __launch_bounds__(kThreads) void gla_scan_kernel(
     const int row = w + 4 * r;
     S[r] = has_col && row < dk ? st[static_cast<size_t>(row) * dv + col] : 0.f;
   }
+  const float fixed = decay ? decay[hd] : 0.f;  // one decay for the whole head, given as it is: no exponential
   for (int t = t_begin; t < t_end; ++t) {
     const float* xr = x + static_cast<size_t>(t) * width;
     const float* qr = xr + hd * dk;
@@ -115,7 +116,7 @@ __global__ __launch_bounds__(kThreads) void gla_scan_kernel(
     for (int r = 0; r < DR; ++r) {
       const int row = w + 4 * r;
       if (row < dk) {
-        S[r] = expf(lr[row]) * S[r] + kr[row] * v;
+        S[r] = (decay ? fixed : expf(lr[row])) * S[r] + kr[row] * v;
         part = fmaf(S[r], qr[row], part);
       }
     }
@@ -325,10 +326,47 @@ __global__ __launch_bounds__(kThreads) void gla_finish_kernel(
       const int e = lane + 64 * u;
       if (e >= dv) continue;
       const float gg = g[hd * dv + e];
-      const float y = v[u] * inv * load_as_float(gain, gain_dt, e) * (gg / (1.f + expf(-gg))) * out_scale;
+      const float y = v[u] * inv * (gain ? load_as_float(gain, gain_dt, e) : 1.f) * (gg / (1.f + expf(-gg))) * out_scale;
       store_from_float(out, out_dt, static_cast<size_t>(n) * out_ld + hd * dv + e, y);
     }
   }
+}
+
+// The rows [q | k | ld | v | g] for a recurrence whose decay is one fixed number per head: the first `rot` elements of
+// every query and key head are turned by position (pairs (e, e + rot / 2), or neighbours (2e, 2e + 1)), the keys then
+// scaled; ld of every key channel of head h is log_decay[h]. One block a token, a thread a pair (or an element).
+__global__ __launch_bounds__(kThreads) void retention_prepare_kernel(
+    const void* __restrict__ proj, int proj_dt, int n_partials, size_t partial_stride, int ld, int col0,
+    const float* __restrict__ log_decay, const float* __restrict__ cos, const float* __restrict__ sin, int rot,
+    int neighbours, const int* __restrict__ positions, float kscale, float* __restrict__ x, int heads, int dk, int dv) {
+  const int n = blockIdx.x, tid = threadIdx.x;
+  const size_t in_row = static_cast<size_t>(n) * ld + col0;
+  const int hk = heads * dk, hv = heads * dv, width = 3 * hk + 2 * hv, half = rot / 2;
+  float* xr = x + static_cast<size_t>(n) * width;
+  auto value = [&](int col) {
+    float v = 0.f;
+    for (int p = 0; p < n_partials; ++p) v += load_as_float(proj, proj_dt, p * partial_stride + in_row + col);
+    return v;
+  };
+  const size_t trig = static_cast<size_t>(positions[n]) * half;
+  // queries (columns 0 .. hk) and keys (hk .. 2 hk): the turned pairs of every head, then the elements that pass
+  for (int i = tid; i < 2 * heads * half; i += kThreads) {
+    const int head = i / half, e = i % half;  // head counts query heads, then key heads
+    const int e1 = neighbours ? 2 * e : e, e2 = neighbours ? 2 * e + 1 : e + half;
+    const int base = head * dk;
+    float a, b;
+    rotate_pair(value(base + e1), value(base + e2), cos[trig + e], sin[trig + e], a, b);
+    const float f = head >= heads ? kscale : 1.f;
+    xr[base + e1] = a * f;
+    xr[base + e2] = b * f;
+  }
+  const int rest = dk - rot;
+  for (int i = tid; i < 2 * heads * rest; i += kThreads) {
+    const int head = i / rest, col = head * dk + rot + i % rest;
+    xr[col] = value(col) * (head >= heads ? kscale : 1.f);
+  }
+  for (int c = tid; c < hk; c += kThreads) xr[2 * hk + c] = log_decay[c / dk];
+  for (int i = tid; i < 2 * hv; i += kThreads) xr[3 * hk + i] = value(2 * hk + i);
 }
 
 }  // namespace
@@ -357,13 +395,13 @@ extern "C" int pyre_gla_prepare(const void* proj, int proj_dt, int n_partials, l
 }
 
 extern "C" int pyre_gla_scan(const float* x, float* state, float* o, const int* q_start, const int* state_slots,
-                             int n_seqs, int heads, int dk, int dv, float qscale, hipStream_t stream) {
+                             int n_seqs, int heads, int dk, int dv, float qscale, const float* decay, hipStream_t stream) {
   PYRE_REQUIRE(heads > 0 && heads <= 65535 && dk > 0 && dk <= 256 && dv > 0, "gla_scan: heads %d, sizes %d / %d are not taken", heads, dk, dv);
   if (n_seqs <= 0) return 0;
   const dim3 grid(n_seqs, heads, (dv + kWave - 1) / kWave);
 #define PYRE_SCAN(DR)                                                                                            \
   hipLaunchKernelGGL(gla_scan_kernel<DR>, grid, dim3(kThreads), 0, stream, x, state, o, q_start, state_slots, heads, \
-                     dk, dv, qscale)
+                     dk, dv, qscale, decay)
   if (dk <= 32) PYRE_SCAN(8);
   else if (dk <= 64) PYRE_SCAN(16);
   else if (dk <= 128) PYRE_SCAN(32);
@@ -408,10 +446,25 @@ extern "C" int pyre_gla_chunks(const float* x, float* scratch, float* state, flo
 
 extern "C" int pyre_gla_finish(const float* o, const float* x, const void* gain, int gain_dt, float eps, float out_scale,
                                void* out, int out_dt, int out_ld, int n, int heads, int dk, int dv, hipStream_t stream) {
-  PYRE_REQUIRE(known_dtype(gain_dt) && known_dtype(out_dt), "gla_finish: bad dtypes");
+  PYRE_REQUIRE((!gain || known_dtype(gain_dt)) && known_dtype(out_dt), "gla_finish: bad dtypes");
   PYRE_REQUIRE(heads > 0 && dk > 0 && dv > 0 && dv <= 256 && eps > 0.f, "gla_finish: sizes %d / %d are not taken", dk, dv);
   if (n <= 0) return 0;
   hipLaunchKernelGGL(gla_finish_kernel, dim3(n), dim3(kThreads), 0, stream, o, x, gain, gain_dt, eps, out_scale, out,
                      out_dt, out_ld, heads, dk, dv);
   return check_launch("gla_finish");
+}
+
+extern "C" int pyre_retention_prepare(const void* proj, int proj_dt, int n_partials, long partial_stride, int ld, int col0,
+                                      const float* log_decay, const float* cos, const float* sin, int rot, int neighbours,
+                                      const int* positions, float kscale, float* x, int n, int heads, int dk, int dv,
+                                      hipStream_t stream) {
+  PYRE_REQUIRE(known_dtype(proj_dt) && n_partials >= 1, "retention_prepare: bad dtypes");
+  PYRE_REQUIRE(heads > 0 && dk > 0 && dv > 0 && log_decay && positions, "retention_prepare: bad sizes");
+  PYRE_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= dk && (rot == 0 || (cos && sin)),
+               "retention_prepare: %d turned elements of a head of %d need tables and an even number", rot, dk);
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(retention_prepare_kernel, dim3(n), dim3(kThreads), 0, stream, proj, proj_dt, n_partials,
+                     static_cast<size_t>(partial_stride), ld, col0, log_decay, cos, sin, rot, neighbours, positions, kscale,
+                     x, heads, dk, dv);
+  return check_launch("retention_prepare");
 }

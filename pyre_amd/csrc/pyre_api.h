@@ -243,14 +243,14 @@ int pyre_attn_biased_tile(const void* q, void* out, int out_ld, int dt, const vo
                           const int* positions, const int* seq_of_token, const int* block_table,
                           int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale,
                           float cap, const float* bias, int far, int window, int keep_first, int chunk,
-                          hipStream_t stream);
+                          const float* sink, int gate_dim, hipStream_t stream);
 // tokens: the n tokens of the flat batch to attend for (null: 0..n-1), a block per token and head.
 int pyre_attn_biased_single(const void* q, void* out, int out_ld, int dt, const void* k_cache,
                             const void* v_cache, const float* gate, float out_scale, const int* tokens,
                             int n, const int* positions, const int* seq_of_token, const int* block_table,
                             int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale,
                             float cap, const float* bias, int far, int window, int keep_first, int chunk,
-                            float* part, int max_spans, hipStream_t stream);
+                            float* part, int max_spans, const float* sink, int gate_dim, hipStream_t stream);
 // part: scratch of n * nq * max_spans * (dv + 2) floats, max_spans = pyre_attn_biased_spans(the most keys a
 // block table holds, window, keep_first): a block then takes one span of 128 keys and a second kernel joins
 // them in their order; null: a block takes all spans of its token and head in turn.
@@ -265,7 +265,8 @@ int pyre_gla_prepare(const void* proj, int proj_dt, int n_partials, long partial
 // state: float32 [slots][heads][dk][dv]; o: float32 [tokens][heads dv]; request s owns the tokens
 // q_start[s] .. q_start[s + 1] - 1 and the slot state_slots[s].
 int pyre_gla_scan(const float* x, float* state, float* o, const int* q_start, const int* state_slots,
-                  int n_seqs, int heads, int dk, int dv, float qscale, hipStream_t stream);
+                  int n_seqs, int heads, int dk, int dv, float qscale, const float* decay,
+                  hipStream_t stream);
 // The same recurrence in chunks of 16 tokens (steps that carry prompt portions); differs from the scan by rounding.
 // scratch: pyre_gla_chunks_scratch(...) floats, starting on 16 bytes; max_tokens: the most tokens that one request brings.
 long pyre_gla_chunks_scratch(int n_tokens, int n_seqs, int heads, int dk, int dv);
@@ -313,4 +314,38 @@ int pyre_route_topk(const void* z, int z_dt, int n_partials, long partial_stride
 int pyre_expert_act(const void* up, int up_dt, int n_partials, long partial_stride, const float* gates, void* out,
                     int out_dt, int n, int experts, int ff, int shared_ff, hipStream_t stream);
 
+// resid += y, out = (out_gain ? RMS(resid) * out_gain : resid): y the sum of up to two pending terms, each with an RMS
+// norm and gain of its own (or none) and a factor, the sum normed again if outer_gain is given (postnorm.hip).
+int pyre_add_rms_terms(float* resid, const void* a, int a_dt, int a_partials, long a_stride, const void* a_gain,
+                       int a_gain_dt, float a_scale, const void* b, int b_dt, int b_partials, long b_stride,
+                       const void* b_gain, int b_gain_dt, float b_scale, float inner_eps, const void* outer_gain,
+                       int outer_dt, float outer_eps, const void* out_gain, int out_gain_dt, float out_eps, void* out,
+                       int out_dt, const int* rows, int n, int hidden, hipStream_t stream);
+
+// out[n] = table[ids[n]] + pairs[row of (previous token, token)]; state [slots][1] float32 holds a request's last token.
+int pyre_bigram_embed(const void* table, const void* pairs, int dt, const int* ids, const int* positions,
+                      const int* seq_of_token, const int* q_start, float* state, const int* state_slots, float* out, int n,
+                      int hidden, int buckets, int mul_prev, int mul_cur, hipStream_t stream);
+
+// The input product of an attention whose projections go through a short causal convolution (conv_attention.hip).
+int pyre_conv_qkv_write(const void* proj, int proj_dt, int n_partials, long partial_stride, int ld, int col0,
+                        const float* taps_w, int taps, float* conv_state, const int* state_slots, const int* seq_of_token,
+                        const int* q_start, int n_seqs, const float* q_gain, const float* k_gain, float eps,
+                        const float* cos, const float* sin, int rot, int neighbours, const int* positions, void* q_out,
+                        int q_dt, void* k_cache, void* v_cache, int cache_dt, float* gate_out, const int* slots, int n,
+                        int nq, int nkv, int dk, int dv, int page_size, int write_kv, hipStream_t stream);
+
+// The rows [q | k | log decay | v | g] of the recurrent kernels for a fixed decay per head, queries and keys turned.
+int pyre_retention_prepare(const void* proj, int proj_dt, int n_partials, long partial_stride, int ld, int col0,
+                           const float* log_decay, const float* cos, const float* sin, int rot, int neighbours,
+                           const int* positions, float kscale, float* x, int n, int heads, int dk, int dv,
+                           hipStream_t stream);
+
+int pyre_route_grouped(const void* z, int z_dt, int n_partials, long partial_stride, const void* bias, int bias_dt,
+                       const float* correction, float* gates, int n, int experts, int top, int groups, int keep_groups,
+                       hipStream_t stream);
+int pyre_expert_glu_act(const void* gu, int gu_dt, int n_partials, long partial_stride, const float* gates,
+                        long gates_stride, void* out, int out_dt, int n, int experts, int ff, hipStream_t stream);
+int pyre_add_weighted_rows(float* p, const void* h, int h_dt, long h_stride, const float* gates, long gates_stride,
+                           int first, int count, int n, int width, hipStream_t stream);
 }  // extern "C"

@@ -285,8 +285,11 @@ class Engine:
         caches it reads), in the order of the layer's descriptions."""
         cache = self.cache
         out = []
-        for pos, call in enumerate(self.model.schedule):
-            src = call.cache_from if call.cache_from is not None else pos
+        entries = [(call.cache_from if call.cache_from is not None else pos, call.cache_from is None)
+                   for pos, call in enumerate(self.model.schedule)]
+        if cache.caches_of_entry(len(entries)):  # what the embedding keeps lies behind the layers' entries
+            entries.append((len(entries), True))
+        for src, writes in entries:
             mine = []
             for k in range(cache.caches_of_entry(src)):
                 kind, gi = cache.group_of_cell[(src, k)]
@@ -295,7 +298,7 @@ class Engine:
                     li = g.layer_index(src, k)
                     mine.append(PagedLayerView({name: t[li] for name, t in g.tensors.items()}, views[f"table{gi}"],
                                                views[f"slots{gi}"], g.page_size, g.spec.window,
-                                               writes=call.cache_from is None))
+                                               writes=writes))
                 else:
                     g = cache.state_groups[gi]
                     mine.append(StateLayerView(g.tensor[g.layer_index(src, k)], views["state_slots"]))

@@ -11,7 +11,7 @@ from ctypes import c_float, c_int, c_long, c_void_p
 
 from pyre_amd.hip import build as _build
 
-ABI_VERSION = 26
+ABI_VERSION = 27
 
 
 class KernelError(RuntimeError):
@@ -59,11 +59,11 @@ _SIGNATURES = {
     "pyre_clipped_glu": [P, I, I, L, P, I, I, I, F, F, F, F, P],
     "pyre_scale": [P, L, F, P],
     "pyre_unit_qkv_write": [P, I, I, L, I, I, P, I, P, P, I, P, P, I, I, I, I, I, I, I, F, I, P],
-    "pyre_attn_biased_tile": [P, P, I, I, P, P, P, F, P, I, P, P, P, I, I, I, I, I, I, F, F, P, I, I, I, I, P],
-    "pyre_attn_biased_single": [P, P, I, I, P, P, P, F, P, I, P, P, P, I, I, I, I, I, I, F, F, P, I, I, I, I, P, I, P],
+    "pyre_attn_biased_tile": [P, P, I, I, P, P, P, F, P, I, P, P, P, I, I, I, I, I, I, F, F, P, I, I, I, I, P, I, P],
+    "pyre_attn_biased_single": [P, P, I, I, P, P, P, F, P, I, P, P, P, I, I, I, I, I, I, F, F, P, I, I, I, I, P, I, P, I, P],
     "pyre_attn_biased_spans": [I, I, I, I],
     "pyre_gla_prepare": [P, I, I, L, I, I, P, I, P, I, F, P, I, I, I, I, I, P],
-    "pyre_gla_scan": [P, P, P, P, P, I, I, I, I, F, P],
+    "pyre_gla_scan": [P, P, P, P, P, I, I, I, I, F, P, P],
     "pyre_gla_chunks": [P, P, P, P, P, P, I, I, I, I, I, I, F, P],
     "pyre_gla_chunks_scratch": [I, I, I, I, I],
     "pyre_gla_finish": [P, P, P, I, F, F, P, I, I, I, I, I, I, P],
@@ -74,6 +74,14 @@ _SIGNATURES = {
     "pyre_head_matmul": [P, I, P, P, I, I, I, I, I, I, P],
     "pyre_route_topk": [P, I, I, L, P, I, P, I, I, I, P],
     "pyre_expert_act": [P, I, I, L, P, P, I, I, I, I, I, P],
+    "pyre_add_rms_terms": [P, P, I, I, L, P, I, F, P, I, I, L, P, I, F, F, P, I, F, P, I, F, P, I, P, I, I, P],
+    "pyre_bigram_embed": [P, P, I, P, P, P, P, P, P, P, I, I, I, I, I, P],
+    "pyre_conv_qkv_write": [P, I, I, L, I, I, P, I, P, P, P, P, I, P, P, F, P, P, I, I, P, P, I, P, P, I, P, P, I, I, I, I,
+                            I, I, I, P],
+    "pyre_retention_prepare": [P, I, I, L, I, I, P, P, P, I, I, P, F, P, I, I, I, I, P],
+    "pyre_route_grouped": [P, I, I, L, P, I, P, P, I, I, I, I, I, P],
+    "pyre_expert_glu_act": [P, I, I, L, P, L, P, I, I, I, I, P],
+    "pyre_add_weighted_rows": [P, P, I, L, P, L, I, I, I, I, P],
 }
 
 _lib = None

@@ -65,11 +65,13 @@ def _ptr(t: torch.Tensor | None) -> int | None:
 
 @dataclass
 class PostNorm:
-    """The norm of a sublayer's own result: LN(term; eps) * gain (* scale), element by element."""
+    """The norm of a sublayer's own result: LN(term; eps) * gain (* scale), element by element (``kind`` "layer"),
+    or term / sqrt(mean(term^2) + eps) * gain (``kind`` "rms")."""
 
     gain: torch.Tensor
     eps: float
     scale: torch.Tensor | None = None
+    kind: str = "layer"
 
 
 @dataclass
@@ -87,6 +89,9 @@ class Partials:
     #: mixer and feed-forward read the same rows hands on both): only a norm that says so takes them
     scale: float = 1.0
     more: "Partials | None" = None
+    #: a norm that the sum of this term and of ``more`` (each after its own norm and factor) goes through before it is
+    #: added: only a norm that says so takes it (:func:`add_rms_terms`)
+    outer: "PostNorm | None" = None
 
     def __post_init__(self) -> None:
         if self.data.dim() != 3 or not self.data.is_contiguous():
@@ -148,7 +153,7 @@ def add_rmsnorm(resid: torch.Tensor, delta: Partials | None, gain: torch.Tensor,
     if delta is not None:
         if delta.rows < resid.shape[0]:
             raise KernelError("add_rmsnorm: delta has fewer rows than the residual")
-        if delta.post is not None or delta.scale != 1.0 or delta.more is not None:
+        if delta.post is not None or delta.scale != 1.0 or delta.more is not None or delta.outer is not None:
             raise KernelError("add_rmsnorm: a term that is normed or scaled before it is added, or comes with another, is not taken")
         d = delta._args(hidden)
     else:
@@ -179,7 +184,8 @@ def add_layernorm(resid: torch.Tensor, delta: Partials | None, gain: torch.Tenso
     if delta is not None:
         if delta.rows < resid.shape[0]:
             raise KernelError("add_layernorm: delta has fewer rows than the residual")
-        if delta.scale != 1.0 or delta.more is not None:
+        if delta.scale != 1.0 or delta.more is not None or delta.outer is not None or \
+                (delta.post is not None and delta.post.kind != "layer"):
             raise KernelError("add_layernorm: a term that is scaled before it is added, or comes with another, is not taken")
         d = delta._args(hidden)
         if delta.post is not None:
@@ -269,8 +275,12 @@ ATTN_BIASED_TILE_MAX_KEY_HEAD = 128  #: the largest key head of the tile kernel 
 
 
 def _attn_biased_common(q, out, k_cache, v_cache, gate, positions, seq_of_token, block_table, bias, far,
-                        nq, nkv, dk, dv, page_size):
-    _dev(q, out, k_cache, v_cache, gate, positions, seq_of_token, block_table, bias)
+                        nq, nkv, dk, dv, page_size, sink=None, gate_dim=1):
+    _dev(q, out, k_cache, v_cache, gate, positions, seq_of_token, block_table, bias, sink)
+    if gate_dim not in (1, dv):
+        raise KernelError("attn_biased: a gate per head or per element of the value head")
+    if sink is not None and (sink.dtype != torch.float32 or not sink.is_contiguous() or sink.numel() != nq):
+        raise KernelError(f"attn_biased: the sinks are contiguous float32 [{nq}]")
     if not (q.dtype == out.dtype == k_cache.dtype == v_cache.dtype):
         raise KernelError("attn_biased: queries, caches and output share one element type")
     if tuple(k_cache.shape[1:]) != (nkv, page_size, dk) or tuple(v_cache.shape[1:]) != (nkv, page_size, dv):
@@ -282,21 +292,25 @@ def _attn_biased_common(q, out, k_cache, v_cache, gate, positions, seq_of_token,
         raise KernelError("attn_biased: block table must be int32 [rows, pages]")
     _i32("positions", positions), _i32("seq_of_token", seq_of_token)
     if gate is not None and (gate.dtype != torch.float32 or not gate.is_contiguous()):
-        raise KernelError("attn_biased: gates are contiguous float32 [N, nq]")
+        raise KernelError("attn_biased: gates are contiguous float32 [N, nq] or [N, nq*dv]")
     if bias is not None and (bias.dtype != torch.float32 or not bias.is_contiguous() or tuple(bias.shape) != (nq, far + 1)):
         raise KernelError(f"attn_biased: the bias by distance is float32 [{nq}, {far + 1}]")
 
 
 def attn_biased_tile(q, out, k_cache, v_cache, gate, out_scale, tiles, n_tiles, positions, seq_of_token,
-                     block_table, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first, chunk: int = 0) -> None:
-    """Prompt portions of the capped, biased attention; ``tiles`` is int32 [n_tiles, 2] = (first token, count <= 32)."""
+                     block_table, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first, chunk: int = 0,
+                     sink: torch.Tensor | None = None, gate_dim: int = 1) -> None:
+    """Prompt portions of the capped, biased attention; ``tiles`` is int32 [n_tiles, 2] = (first token, count <= 32).
+    ``sink`` (float32 [nq]): exp(sink) of the head joins the softmax's denominator, a key without a value.
+    ``gate_dim`` = dv: ``gate`` is [N, nq*dv], a gate per element of the output."""
     _attn_biased_common(q, out, k_cache, v_cache, gate, positions, seq_of_token, block_table, bias, far,
-                        nq, nkv, dk, dv, page_size)
+                        nq, nkv, dk, dv, page_size, sink, gate_dim)
     _i32("tiles", tiles, 2 * n_tiles)
     call("pyre_attn_biased_tile", q.data_ptr(), out.data_ptr(), out.stride(0), dtype_code(q), k_cache.data_ptr(),
          v_cache.data_ptr(), _ptr(gate), float(out_scale), tiles.data_ptr(), n_tiles, positions.data_ptr(),
          seq_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0), nq, nkv, dk, dv, page_size,
-         float(scale), float(cap), _ptr(bias), int(far), int(window), int(keep_first), int(chunk), _stream())
+         float(scale), float(cap), _ptr(bias), int(far), int(window), int(keep_first), int(chunk), _ptr(sink),
+         int(gate_dim), _stream())
 
 
 def attn_biased_spans(table_width: int, page_size: int, window: int, keep_first: int, chunk: int = 0) -> int:
@@ -308,12 +322,14 @@ def attn_biased_spans(table_width: int, page_size: int, window: int, keep_first:
 
 def attn_biased_single(q, out, k_cache, v_cache, gate, out_scale, tokens, n, positions, seq_of_token,
                        block_table, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first,
-                       scratch: torch.Tensor | None = None, chunk: int = 0) -> None:
+                       scratch: torch.Tensor | None = None, chunk: int = 0, sink: torch.Tensor | None = None,
+                       gate_dim: int = 1) -> None:
     """The same for ``n`` tokens one by one (``tokens``: which of the flat batch, None: the first n). ``scratch``
     (float32, ``n * nq * attn_biased_spans(...) * (dv + 2)`` elements): a block per span of 128 keys and a second
-    kernel that joins them, instead of a block per token and head that takes its spans in turn."""
+    kernel that joins them, instead of a block per token and head that takes its spans in turn. ``sink`` and
+    ``gate_dim`` as for :func:`attn_biased_tile`."""
     _attn_biased_common(q, out, k_cache, v_cache, gate, positions, seq_of_token, block_table, bias, far,
-                        nq, nkv, dk, dv, page_size)
+                        nq, nkv, dk, dv, page_size, sink, gate_dim)
     if tokens is not None:
         _dev(tokens), _i32("tokens", tokens, n)
     spans = 0
@@ -325,7 +341,8 @@ def attn_biased_single(q, out, k_cache, v_cache, gate, out_scale, tokens, n, pos
     call("pyre_attn_biased_single", q.data_ptr(), out.data_ptr(), out.stride(0), dtype_code(q), k_cache.data_ptr(),
          v_cache.data_ptr(), _ptr(gate), float(out_scale), _ptr(tokens), n, positions.data_ptr(),
          seq_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0), nq, nkv, dk, dv, page_size,
-         float(scale), float(cap), _ptr(bias), int(far), int(window), int(keep_first), int(chunk), _ptr(scratch), spans, _stream())
+         float(scale), float(cap), _ptr(bias), int(far), int(window), int(keep_first), int(chunk), _ptr(scratch), spans,
+         _ptr(sink), int(gate_dim), _stream())
 
 
 GLA_MAX_RANK = 512     #: the widest low-rank input of the decay (linear_attention.hip)
@@ -366,13 +383,17 @@ def gla_chunks_scratch(n_tokens: int, n_seqs: int, heads: int, dk: int, dv: int)
 
 def gla_scan(x: torch.Tensor, state: torch.Tensor, o: torch.Tensor, q_start: torch.Tensor, state_slots: torch.Tensor,
              n_seqs: int, heads: int, dk: int, dv: int, qscale: float, chunks: torch.Tensor | None = None,
-             max_tokens: int = 0) -> None:
+             max_tokens: int = 0, decay: torch.Tensor | None = None) -> None:
     """The recurrence over each request's tokens of the step, from and into ``state [slots, heads, dk, dv]``;
     ``o`` (float32 [N, heads*dv]) receives qscale * S^T q. ``chunks``: scratch (float32,
     :func:`gla_chunks_scratch` elements) that makes the walk take sixteen tokens at a time on the matrix cores
     (for steps that carry prompt portions, ``max_tokens`` the most that one request brings; the token-by-token
-    walk is the one for single tokens): a difference of rounding."""
-    _dev(x, state, o, q_start, state_slots, chunks)
+    walk is the one for single tokens): a difference of rounding. ``decay`` (float32 [heads]): the token-by-token walk
+    multiplies head h's state by decay[h] itself instead of by the exponential of the rows' logarithms (which must be its
+    logarithm all the same: the walk in chunks goes by them)."""
+    _dev(x, state, o, q_start, state_slots, chunks, decay)
+    if decay is not None and (decay.dtype != torch.float32 or decay.numel() != heads or not decay.is_contiguous()):
+        raise KernelError("gla_scan: one float32 decay per head")
     for name, t in (("x", x), ("state", state), ("o", o)):
         if t.dtype != torch.float32 or not t.is_contiguous():
             raise KernelError(f"gla_scan: {name} is contiguous float32")
@@ -381,7 +402,7 @@ def gla_scan(x: torch.Tensor, state: torch.Tensor, o: torch.Tensor, q_start: tor
     _i32("q_start", q_start, n_seqs + 1), _i32("state_slots", state_slots, n_seqs)
     if chunks is None:
         call("pyre_gla_scan", x.data_ptr(), state.data_ptr(), o.data_ptr(), q_start.data_ptr(), state_slots.data_ptr(),
-             n_seqs, heads, dk, dv, float(qscale), _stream())
+             n_seqs, heads, dk, dv, float(qscale), _ptr(decay), _stream())
         return
     n = o.shape[0]
     if chunks.dtype != torch.float32 or not chunks.is_contiguous() or chunks.numel() < gla_chunks_scratch(n, n_seqs, heads, dk, dv):
@@ -390,16 +411,17 @@ def gla_scan(x: torch.Tensor, state: torch.Tensor, o: torch.Tensor, q_start: tor
          state_slots.data_ptr(), n, n_seqs, int(max_tokens), heads, dk, dv, float(qscale), _stream())
 
 
-def gla_finish(o: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, eps: float, out_scale: float, out: torch.Tensor,
+def gla_finish(o: torch.Tensor, x: torch.Tensor, gain: torch.Tensor | None, eps: float, out_scale: float, out: torch.Tensor,
                n: int, heads: int, dk: int, dv: int) -> None:
-    """out[n, h*dv + e] = o / rms(o over dv) * gain[e] * silu(g) * out_scale; ``out`` has contiguous rows."""
+    """out[n, h*dv + e] = o / rms(o over dv) * gain[e] * silu(g) * out_scale (``gain`` None: ones); ``out`` has contiguous rows."""
     _dev(o, x, gain, out)
     if o.dtype != torch.float32 or x.dtype != torch.float32 or not o.is_contiguous() or not x.is_contiguous():
         raise KernelError("gla_finish: o and x are contiguous float32")
-    if gain.numel() != dv or out.dim() != 2 or out.stride(1) != 1 or out.shape[1] < heads * dv or out.shape[0] < n:
+    if (gain is not None and gain.numel() != dv) or out.dim() != 2 or out.stride(1) != 1 or out.shape[1] < heads * dv or out.shape[0] < n:
         raise KernelError("gla_finish: gain [dv] and out [>= n, >= heads*dv] expected")
-    _contig("gain", gain)
-    call("pyre_gla_finish", o.data_ptr(), x.data_ptr(), gain.data_ptr(), dtype_code(gain), float(eps), float(out_scale),
+    if gain is not None:
+        _contig("gain", gain)
+    call("pyre_gla_finish", o.data_ptr(), x.data_ptr(), _ptr(gain), dtype_code(gain) if gain is not None else 0, float(eps), float(out_scale),
          out.data_ptr(), dtype_code(out), out.stride(0), n, heads, dk, dv, _stream())
 
 
@@ -986,7 +1008,7 @@ def add_tanhnorm(resid: torch.Tensor, delta: Partials | None, alpha: torch.Tenso
     while t is not None:
         if t.rows < resid.shape[0]:
             raise KernelError("add_tanhnorm: a pending term has fewer rows than the residual")
-        if t.post is not None:
+        if t.post is not None or t.outer is not None:
             raise KernelError("add_tanhnorm: a term that is to be normed before it is added is not taken")
         terms.append((*t._args(hidden), float(t.scale)))
         t = t.more
@@ -1121,3 +1143,246 @@ def expert_act(up: Partials, gates: torch.Tensor, out: torch.Tensor, n: int, exp
     _contig("out", out)
     call("pyre_expert_act", up.data.data_ptr(), dtype_code(up.data), up.count, up.stride, gates.data_ptr(),
          out.data_ptr(), dtype_code(out), n, experts, ff, shared_ff, _stream())
+
+
+def _term_args(t: Partials | None, hidden: int, what: str):
+    """(data, dtype, count, stride, own gain, its dtype, factor) of one pending term of :func:`add_rms_terms`."""
+    if t is None:
+        return (None, 0, 0, 0, None, 0, 1.0), None
+    if t.bias is not None:
+        raise KernelError(f"{what}: a pending bias is not taken")
+    if t.width != hidden:
+        raise KernelError(f"{what}: a pending term is {t.width} wide, {hidden} expected")
+    gain = None
+    if t.post is not None:
+        if t.post.kind != "rms" or t.post.scale is not None:
+            raise KernelError(f"{what}: a term's own norm must be an RMS norm without a layer scale")
+        gain = t.post.gain
+        _dev(gain), _contig("post.gain", gain)
+        if gain.numel() != hidden:
+            raise KernelError(f"{what}: a term's gain does not fit the residual")
+    return (t.data.data_ptr(), dtype_code(t.data), t.count, t.stride, _ptr(gain),
+            dtype_code(gain) if gain is not None else 0, float(t.scale)), t.post
+
+
+def add_rms_terms(resid: torch.Tensor, delta: Partials | None, gain: torch.Tensor | None, eps: float,
+                  out: torch.Tensor | None, rows: torch.Tensor | None = None) -> None:
+    """resid += y; out = gain is None ? resid : resid / sqrt(mean(resid^2) + eps) * gain, rounded to ``out``'s type.
+
+    y is the pending term: up to two terms (``delta`` and ``delta.more``), each the sum of its partial sums, divided by
+    its root mean square and times its gain if it carries a norm of its own (``post``, kind "rms"), times its factor
+    (``scale``); their sum goes through ``delta.outer`` (an RMS norm again) if that is given. With ``rows`` only those
+    rows are handled, into ``out[0:len(rows)]``, and ``resid`` is left as it was."""
+    _dev(resid, gain, out, rows)
+    hidden = resid.shape[-1]
+    if resid.dtype != torch.float32 or resid.dim() != 2:
+        raise KernelError("add_rms_terms: the residual stream is float32 [N, H]")
+    _contig("resid", resid)
+    n = resid.shape[0] if rows is None else rows.numel()
+    if out is not None:
+        if out.shape[-1] != hidden or out.shape[0] < n:
+            raise KernelError("add_rms_terms: out does not fit the residual")
+        _contig("out", out)
+    if gain is not None:
+        if out is None or gain.numel() != hidden:
+            raise KernelError("add_rms_terms: the output norm's gain does not fit the residual")
+        _contig("gain", gain)
+    if rows is not None:
+        _i32("rows", rows)
+    more = delta.more if delta is not None else None
+    if more is not None and (more.more is not None or more.outer is not None):
+        raise KernelError("add_rms_terms: at most two pending terms, the norm of their sum on the first")
+    for t in (delta, more):
+        if t is not None and t.rows < resid.shape[0]:
+            raise KernelError("add_rms_terms: a pending term has fewer rows than the residual")
+    a, post_a = _term_args(delta, hidden, "add_rms_terms")
+    b, post_b = _term_args(more, hidden, "add_rms_terms")
+    inner = [p.eps for p in (post_a, post_b) if p is not None]
+    if len(set(inner)) > 1:
+        raise KernelError("add_rms_terms: the terms' own norms share one eps")
+    outer = delta.outer if delta is not None else None
+    o = (None, 0, 0.0)
+    if outer is not None:
+        if outer.kind != "rms" or outer.scale is not None or outer.gain.numel() != hidden:
+            raise KernelError("add_rms_terms: the norm of the sum is an RMS norm with a gain over the hidden size")
+        _dev(outer.gain), _contig("outer.gain", outer.gain)
+        o = (outer.gain.data_ptr(), dtype_code(outer.gain), float(outer.eps))
+    call("pyre_add_rms_terms", resid.data_ptr(), *a, *b, float(inner[0]) if inner else 0.0, *o, _ptr(gain),
+         dtype_code(gain) if gain is not None else 0, float(eps), _ptr(out), dtype_code(out) if out is not None else 0,
+         _ptr(rows), n, hidden, _stream())
+
+
+def bigram_embed(table: torch.Tensor, pairs: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor,
+                 seq_of_token: torch.Tensor, q_start: torch.Tensor, state: torch.Tensor, state_slots: torch.Tensor,
+                 out: torch.Tensor, buckets: int, mul_prev: int, mul_cur: int) -> None:
+    """out[n] = float32(table[ids[n]]) + float32(pairs[row]), row = (previous token * mul_prev + ids[n] * mul_cur) mod
+    buckets, or ``buckets`` at position 0. The previous token of a request's first token of the step is
+    ``state[slot, 0]`` (float32, an integer value), which then takes the request's last token of the step."""
+    _dev(table, pairs, ids, positions, seq_of_token, q_start, state, state_slots, out)
+    n, hidden = out.shape
+    if table.dim() != 2 or table.shape[1] != hidden or out.dtype != torch.float32 or table.dtype != pairs.dtype:
+        raise KernelError("bigram_embed: tables [V, H] / [buckets + 1, H] of one type and float32 out [N, H] expected")
+    if tuple(pairs.shape) != (buckets + 1, hidden) or buckets <= 0 or mul_prev < 0 or mul_cur < 0:
+        raise KernelError(f"bigram_embed: the pair table is [{buckets + 1}, {hidden}]")
+    if state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 2 or state.shape[1] != 1:
+        raise KernelError("bigram_embed: the state is contiguous float32 [slots, 1]")
+    _contig("table", table), _contig("pairs", pairs), _contig("out", out)
+    _i32("ids", ids, n), _i32("positions", positions, n), _i32("seq_of_token", seq_of_token, n)
+    _i32("q_start", q_start), _i32("state_slots", state_slots)
+    call("pyre_bigram_embed", table.data_ptr(), pairs.data_ptr(), dtype_code(table), ids.data_ptr(), positions.data_ptr(),
+         seq_of_token.data_ptr(), q_start.data_ptr(), state.data_ptr(), state_slots.data_ptr(), out.data_ptr(), n, hidden,
+         int(buckets), int(mul_prev), int(mul_cur), _stream())
+
+
+CONV_MAX_TAPS = 16  #: the most taps of the short convolution (conv_attention.hip)
+
+
+def conv_qkv_write(proj: Partials, col0: int, taps_w: torch.Tensor | None, conv_state: torch.Tensor | None,
+                   state_slots: torch.Tensor, seq_of_token: torch.Tensor, q_start: torch.Tensor, n_seqs: int,
+                   q_gain: torch.Tensor | None, k_gain: torch.Tensor | None, eps: float, cos: torch.Tensor | None,
+                   sin: torch.Tensor | None, rot: int, neighbours: bool, positions: torch.Tensor, q_out: torch.Tensor,
+                   k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, gate_out: torch.Tensor | None,
+                   slots: torch.Tensor | None, n: int, nq: int, nkv: int, dk: int, dv: int, page_size: int) -> None:
+    """Finish a step's input product from column ``col0`` on (``nq`` query and ``nkv`` key heads of ``dk``, ``nkv`` value
+    heads of ``dv``, then ``nq * dv`` gate columns if ``gate_out`` is given). Queries, keys and values first go through a
+    causal convolution over the request's tokens, ``taps_w`` float32 [channels, taps] (None: none), whose inputs before
+    the step's first token come from ``conv_state`` (float32 [slots, taps - 1, channels], the request's last projected
+    rows; it is brought up to date after every token has read it). Then queries and keys are divided by their root mean
+    square per head, times ``q_gain`` / ``k_gain`` over ``dk`` (None: not normed), and their first ``rot`` elements turned
+    by position (``neighbours``: element 2e with 2e + 1, else e with e + rot/2). Queries go to ``q_out [N, nq*dk]``, keys and
+    values to their pages at ``slots``, sigmoid(gate) to float32 ``gate_out [N, nq*dv]``."""
+    _dev(proj.data, taps_w, conv_state, state_slots, seq_of_token, q_start, q_gain, k_gain, cos, sin, positions, q_out,
+         k_cache, v_cache, gate_out, slots)
+    channels = (nq + nkv) * dk + nkv * dv
+    args = _proj_args(proj, col0, channels + (nq * dv if gate_out is not None else 0))
+    if proj.rows < n or q_out.numel() < n * nq * dk:
+        raise KernelError("conv_qkv_write: buffers are smaller than the batch")
+    _contig("q_out", q_out), _i32("positions", positions, n), _i32("seq_of_token", seq_of_token, n)
+    _i32("q_start", q_start, n_seqs + 1), _i32("state_slots", state_slots, n_seqs)
+    taps = 0
+    if taps_w is not None:
+        taps = taps_w.shape[1]
+        if taps_w.dtype != torch.float32 or not taps_w.is_contiguous() or tuple(taps_w.shape) != (channels, taps) or \
+                not (1 <= taps <= CONV_MAX_TAPS):
+            raise KernelError(f"conv_qkv_write: the taps are contiguous float32 [{channels}, 1..{CONV_MAX_TAPS}]")
+        if taps > 1:
+            if conv_state is None or conv_state.dtype != torch.float32 or not conv_state.is_contiguous() or \
+                    tuple(conv_state.shape[1:]) != (taps - 1, channels):
+                raise KernelError(f"conv_qkv_write: the state is contiguous float32 [slots, {taps - 1}, {channels}]")
+    for name, g in (("q_gain", q_gain), ("k_gain", k_gain)):
+        if g is not None and (g.dtype != torch.float32 or g.numel() != dk or not g.is_contiguous()):
+            raise KernelError(f"conv_qkv_write: {name} is contiguous float32 [{dk}]")
+    if (q_gain is None) != (k_gain is None):
+        raise KernelError("conv_qkv_write: queries and keys are normed together or not at all")
+    if rot:
+        if rot % 2 or rot > dk or cos is None or sin is None or cos.dtype != torch.float32 or sin.dtype != torch.float32 \
+                or cos.dim() != 2 or cos.shape[1] != rot // 2 or tuple(cos.shape) != tuple(sin.shape):
+            raise KernelError("conv_qkv_write: cos and sin are float32 [positions, rot / 2], rot even and within the head")
+        _contig("cos", cos), _contig("sin", sin)
+    write = k_cache is not None
+    cache_dt = dtype_code(q_out)
+    if write:
+        if v_cache is None or slots is None:
+            raise KernelError("conv_qkv_write: k cache without v cache or slots")
+        _i32("slots", slots, n), _contig("k_cache", k_cache), _contig("v_cache", v_cache)
+        if tuple(k_cache.shape[1:]) != (nkv, page_size, dk) or tuple(v_cache.shape[1:]) != (nkv, page_size, dv) \
+                or k_cache.dtype != v_cache.dtype:
+            raise KernelError(f"conv_qkv_write: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} do not fit "
+                              f"nkv={nkv} page={page_size} dk={dk} dv={dv}")
+        cache_dt = dtype_code(k_cache)
+    if gate_out is not None and (gate_out.dtype != torch.float32 or gate_out.numel() < n * nq * dv or not gate_out.is_contiguous()):
+        raise KernelError("conv_qkv_write: gates are contiguous float32 [N, nq*dv]")
+    call("pyre_conv_qkv_write", *args, _ptr(taps_w), taps, _ptr(conv_state) if taps > 1 else None, state_slots.data_ptr(),
+         seq_of_token.data_ptr(), q_start.data_ptr(), n_seqs, _ptr(q_gain), _ptr(k_gain), float(eps),
+         _ptr(cos) if rot else None, _ptr(sin) if rot else None, int(rot), int(bool(neighbours)), positions.data_ptr(),
+         q_out.data_ptr(), dtype_code(q_out), _ptr(k_cache), _ptr(v_cache), cache_dt, _ptr(gate_out), _ptr(slots), n, nq,
+         nkv, dk, dv, page_size, 1 if write else 0, _stream())
+
+
+def retention_prepare(proj: Partials, col0: int, log_decay: torch.Tensor, cos: torch.Tensor | None,
+                      sin: torch.Tensor | None, rot: int, neighbours: bool, positions: torch.Tensor, kscale: float,
+                      x: torch.Tensor, n: int, heads: int, dk: int, dv: int) -> None:
+    """Finish the input product from column ``col0`` on (q, k: heads*dk each; v, g: heads*dv each) into the float32 rows
+    [q | k | log decay | v | g] that the recurrent kernels share: the first ``rot`` elements of every query and key head
+    turned by position, the keys then times ``kscale``; every key channel of head h gets ``log_decay[h]``."""
+    _dev(proj.data, log_decay, cos, sin, positions, x)
+    args = _proj_args(proj, col0, 2 * heads * dk + 2 * heads * dv)
+    if log_decay.dtype != torch.float32 or log_decay.numel() != heads or not log_decay.is_contiguous():
+        raise KernelError("retention_prepare: one float32 logarithm of a decay per head")
+    if x.dtype != torch.float32 or not x.is_contiguous() or x.shape[-1] != gla_row_width(heads, dk, dv) or x.shape[0] < n \
+            or proj.rows < n:
+        raise KernelError("retention_prepare: x is contiguous float32 [>= n, 3*heads*dk + 2*heads*dv]")
+    _i32("positions", positions, n)
+    if rot:
+        if rot % 2 or rot > dk or cos is None or sin is None or cos.dtype != torch.float32 or sin.dtype != torch.float32 \
+                or cos.dim() != 2 or cos.shape[1] != rot // 2 or tuple(cos.shape) != tuple(sin.shape):
+            raise KernelError("retention_prepare: cos and sin are float32 [positions, rot / 2], rot even and within the head")
+        _contig("cos", cos), _contig("sin", sin)
+    call("pyre_retention_prepare", *args, log_decay.data_ptr(), _ptr(cos) if rot else None, _ptr(sin) if rot else None,
+         int(rot), int(bool(neighbours)), positions.data_ptr(), float(kscale), x.data_ptr(), n, heads, dk, dv, _stream())
+
+
+def route_grouped(z: Partials, correction: torch.Tensor | None, gates: torch.Tensor, n: int, top: int, groups: int,
+                  keep_groups: int) -> None:
+    """gates[n, e] (float32 [N, experts]) = s_e for the ``top`` experts of largest s_e + correction_e among the experts
+    of the ``keep_groups`` of ``groups`` equal groups of neighbours whose largest such number is largest (the lower index
+    among equals, of groups as of experts), 0 for the others; s = softmax(z) over all experts, ``z`` the router product's
+    partial sums."""
+    _dev(z.data, z.bias, correction, gates)
+    experts = z.width
+    if gates.dtype != torch.float32 or not gates.is_contiguous() or gates.dim() != 2 or gates.shape[1] != experts or \
+            gates.shape[0] < n or z.rows < n:
+        raise KernelError("route_grouped: gates are contiguous float32 [>= n, experts]")
+    if not (0 < experts <= ROUTE_MAX_EXPERTS) or groups <= 0 or experts % groups or not (0 < keep_groups <= groups) or \
+            not (0 < top <= keep_groups * (experts // groups)):
+        raise KernelError(f"route_grouped: {top} of {experts} experts in {keep_groups} of {groups} groups is not a choice "
+                          "this kernel makes")
+    if correction is not None and (correction.dtype != torch.float32 or correction.numel() != experts or
+                                   not correction.is_contiguous()):
+        raise KernelError("route_grouped: the correction is contiguous float32 [experts]")
+    call("pyre_route_grouped", *z._args(experts), _ptr(correction), gates.data_ptr(), n, experts, int(top), int(groups),
+         int(keep_groups), _stream())
+
+
+def expert_glu_act(gu: Partials, gates: torch.Tensor, out: torch.Tensor, n: int, experts: int, ff: int) -> None:
+    """out[n, e*ff + j] = gates[n, e] * silu(g) * u with g = gu[n, e*ff + j] and u = gu[n, experts*ff + e*ff + j]: the
+    experts' gated units, weighted (``gates [N, >= experts]`` with contiguous rows; columns of an expert that the token
+    does not take are not read and written as zero)."""
+    _dev(gu.data, gates, out)
+    width = experts * ff
+    if gu.bias is not None:
+        raise KernelError("expert_glu_act: a pending bias is not supported")
+    if gu.width != 2 * width or gu.rows < n or out.shape[-1] != width or out.shape[0] < n:
+        raise KernelError("expert_glu_act: the product's width does not fit 2 * experts * ff")
+    if gates.dtype != torch.float32 or gates.dim() != 2 or gates.stride(1) != 1 or gates.shape[1] < experts or gates.shape[0] < n:
+        raise KernelError("expert_glu_act: gates are float32 [>= n, >= experts] with contiguous rows")
+    _contig("out", out)
+    call("pyre_expert_glu_act", gu.data.data_ptr(), dtype_code(gu.data), gu.count, gu.stride, gates.data_ptr(),
+         gates.stride(0), out.data_ptr(), dtype_code(out), n, experts, ff, _stream())
+
+
+def add_weighted_rows(p: Partials, h: torch.Tensor, gates: torch.Tensor, first: int, count: int, n: int) -> None:
+    """p[0][n, :] += (gates[n, first] + ... + gates[n, first + count - 1]) * h[n, :]: experts that hand their input back,
+    added to the first partial sum (float32) of the experts' product."""
+    _dev(p.data, h, gates)
+    if p.data.dtype != torch.float32 or p.bias is not None:
+        raise KernelError("add_weighted_rows: float32 partial sums without a bias expected")
+    if h.dim() != 2 or h.shape[1] != p.width or h.stride(1) != 1 or h.shape[0] < n or p.rows < n:
+        raise KernelError("add_weighted_rows: h [>= n, width] with contiguous rows expected")
+    if gates.dtype != torch.float32 or gates.dim() != 2 or gates.stride(1) != 1 or first < 0 or count <= 0 or \
+            first + count > gates.shape[1] or gates.shape[0] < n:
+        raise KernelError("add_weighted_rows: gates are float32 [>= n, >= first + count] with contiguous rows")
+    call("pyre_add_weighted_rows", p.data.data_ptr(), h.data_ptr(), dtype_code(h), h.stride(0), gates.data_ptr(),
+         gates.stride(0), int(first), int(count), n, p.width, _stream())
+
+
+def relu2(up: Partials, out: torch.Tensor, n: int) -> None:
+    """out[n, j] = max(up[n, j], 0)^2, the partial sums added first."""
+    _dev(up.data, out)
+    if up.bias is not None:
+        raise KernelError("relu2: a pending bias is not supported")
+    if up.rows < n or out.shape[-1] != up.width or out.shape[0] < n:
+        raise KernelError("relu2: the output does not fit the product")
+    _contig("out", out)
+    call("pyre_expert_act", up.data.data_ptr(), dtype_code(up.data), up.count, up.stride, None,
+         out.data_ptr(), dtype_code(out), n, 0, 4, up.width, _stream())

@@ -288,12 +288,19 @@ class RMSNormSpec:
     hidden_size: int
     eps: float
     prefix: str                      #: tensor name is ``prefix + ".weight"``
+    name: str | None = None          #: or this, as it stands
     kind: ClassVar[str] = "rmsnorm"
+
+    @property
+    def tensor(self) -> str:
+        return self.name if self.name is not None else f"{self.prefix}.weight"
 
 
 @dataclass(frozen=True)
 class RotarySpec:
-    """Half-split rotary positions: element j pairs with j + rotary_dim/2."""
+    """Rotary positions: element j pairs with j + rotary_dim/2 (``pairing`` "halves"), or element 2j with 2j + 1
+    ("neighbours": a mixer whose kernels turn such pairs says so); the angle of pair j is position * theta^(-2j/d)
+    either way, so the tables are the same."""
 
     head_dim: int
     theta: float
@@ -302,6 +309,7 @@ class RotarySpec:
     #: angles position * theta^(-2j/d) formed in float64 and their cosines and sines rounded to float32 once,
     #: instead of float32 arithmetic all the way
     exact: bool = False
+    pairing: str = "halves"
     kind: ClassVar[str] = "rotary"
 
 
@@ -457,6 +465,93 @@ class SigmoidMoESpec:
 
 
 @dataclass(frozen=True)
+class SinkAttentionSpec:
+    """Grouped softmax attention over a window whose denominator holds one more term, exp(sink) of a learned number
+    per head that has no key and no value (``sink``). Before anything else the projected queries, keys and values go
+    through a causal convolution over time, ``conv_taps`` taps per channel (0: none), whose last ``conv_taps - 1``
+    inputs a request keeps as state; queries and keys are then divided by their root mean square per head, times a
+    gain over ``key_dim`` that the heads share (``qk_norm``), and turned by position (``position``: either pairing).
+    The heads' outputs are multiplied element by element with sigmoid(G h) (``gated``). Tensors: ``prefix + .q / .k /
+    .v / .g / .o / .sink / .q.norm / .k.norm / .q.conv / .k.conv / .v.conv``."""
+
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    key_dim: int
+    value_dim: int
+    scale: float
+    position: Any
+    prefix: str
+    window: int = 0
+    conv_taps: int = 0
+    qk_norm: bool = True
+    norm_eps: float = 1e-6
+    sink: bool = True
+    gated: bool = True
+    kind: ClassVar[str] = "sink_attention"
+
+
+@dataclass(frozen=True)
+class RetentionSpec:
+    """Linear attention with one fixed decay per head: S <- decay_h S + k v^T, o = S^T q with S [key_dim, value_dim]
+    float32 per head and request, no softmax and no denominator. Queries and keys are turned by position
+    (``position``: either pairing), the keys then scaled by key_dim^-1/2. Every head's o is divided by its root mean
+    square (no gain), times silu(G h). Tensors: ``prefix + .q / .k / .v / .g / .o``."""
+
+    hidden_size: int
+    num_heads: int
+    key_dim: int
+    value_dim: int
+    decay: tuple
+    position: Any
+    prefix: str
+    norm_eps: float = 1e-6
+    kind: ClassVar[str] = "retention"
+
+
+@dataclass(frozen=True)
+class ReluSquaredMLPSpec:
+    """down(relu(up(x))^2), no biases. Tensors: ``prefix + .up / .down``."""
+
+    hidden_size: int
+    intermediate_size: int
+    prefix: str
+    kind: ClassVar[str] = "relu2_mlp"
+
+
+@dataclass(frozen=True)
+class GroupedSoftmaxMoESpec:
+    """A mixture of ``experts`` gated units down(silu(gate(x)) * up(x)) of ``expert_size`` hidden units and ``identity``
+    further experts that hand their input back as it is (they own no tensors; the router's last outputs are theirs).
+    Scores s = softmax(router(x)) over all of them; the choice goes by s + a learned correction per expert, among the
+    experts of the ``keep_groups`` of ``groups`` equal groups of neighbours whose largest such number is largest; the
+    ``top`` chosen experts are weighted by s itself, not renormalised. Tensors: ``prefix + .router / .correction``,
+    ``.e<i>.gate / .up / .down``."""
+
+    hidden_size: int
+    experts: int
+    top: int
+    expert_size: int
+    prefix: str
+    identity: int = 0
+    groups: int = 1
+    keep_groups: int = 1
+    kind: ClassVar[str] = "grouped_softmax_moe"
+
+
+@dataclass(frozen=True)
+class PostNormBlockSpec:
+    """x += post_norm(mixer(x)); x += post_norm(feed_forward(x)): the sublayers read the residual stream itself (in the
+    engine's element type) and only their results are normed (RMS norms). ``feed_forward`` None: the first half alone."""
+
+    mixer: Any
+    mixer_post_norm: Any
+    feed_forward: Any = None
+    feed_forward_post_norm: Any = None
+    kind: ClassVar[str] = "post_norm"
+
+
+@dataclass(frozen=True)
 class ParallelBlockSpec:
     """x += scale * (mixer(norm(x)) + feed_forward(norm(x))): one norm, both sublayers read its rows
     (``feed_forward`` None: the mixer alone)."""
@@ -470,11 +565,15 @@ class ParallelBlockSpec:
 
 @dataclass(frozen=True)
 class ParallelMixerSpec:
-    """sum_i scales[i] * branches[i](h): mixers side by side that read the same rows."""
+    """sum_i scales[i] * branches[i](h): mixers side by side that read the same rows. ``out_norms``: every branch's
+    result is first divided by its root mean square over the hidden size (``norm_eps``), times a gain of its own
+    (the tensors named here, one per branch); the branches then keep their output products apart."""
 
     hidden_size: int
     branches: tuple
     scales: tuple
+    out_norms: tuple | None = None
+    norm_eps: float = 1e-6
     kind: ClassVar[str] = "parallel"
 
 
@@ -534,6 +633,21 @@ class EmbeddingSpec:
     hidden_size: int
     name: str = "model.embed_tokens.weight"
     kind: ClassVar[str] = "embedding"
+
+
+@dataclass(frozen=True)
+class BigramEmbeddingSpec:
+    """table[token] + pairs[(previous token * mul_prev + token * mul_cur) mod buckets]; a request's first token
+    takes row ``buckets`` of ``pairs`` (its last). The previous token is state that a request keeps."""
+
+    vocab_size: int
+    hidden_size: int
+    buckets: int
+    mul_prev: int
+    mul_cur: int
+    name: str = "embed"
+    pairs_name: str = "bigram"
+    kind: ClassVar[str] = "bigram_embedding"
 
 
 @dataclass(frozen=True)

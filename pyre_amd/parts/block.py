@@ -7,7 +7,8 @@ from dataclasses import dataclass
 import torch
 
 from pyre_amd.hip.ops import Partials, PostNorm
-from pyre_amd.parts.base import Block, BlockSpec, ParallelBlockSpec, SandwichBlockSpec, TensorSpec, make_part, take
+from pyre_amd.parts.base import (Block, BlockSpec, ParallelBlockSpec, PostNormBlockSpec, SandwichBlockSpec, TensorSpec,
+                                 make_part, take)
 
 
 @dataclass
@@ -170,3 +171,60 @@ class ParallelBlock(Block):
             fed = self.feed_forward.forward(ctx, h)
             more = Partials(fed.data, fed.bias, scale=self.spec.scale)
         state.pending = Partials(mixed.data, mixed.bias, scale=self.spec.scale, more=more)
+
+
+class PostNormBlock(Block):
+    """x += post1(mixer(x)); x += post2(feed_forward(x)) with RMS norms: the sublayers read the residual stream itself,
+    rounded to the engine's element type, and only what they return is normed. No norm runs as a kernel of its own: a
+    sublayer's result is handed on as the pending term with its norm (``Partials.outer``: the norm of the sum of the
+    term's parts, which a mixer of several branches may have normed and scaled one by one), and the kernel that adds
+    it also writes the rows that the next sublayer reads. A layer without a feed-forward is the first half alone."""
+
+    def __init__(self, spec: PostNormBlockSpec):
+        self.spec = spec
+        self.mixer = make_part("mixer", spec.mixer)
+        self.mixer_post = make_part("norm", spec.mixer_post_norm)
+        self.feed_forward = self.feed_forward_post = None
+        if spec.feed_forward is not None:
+            self.feed_forward = make_part("feed_forward", spec.feed_forward)
+            self.feed_forward_post = make_part("norm", spec.feed_forward_post_norm)
+
+    def parts(self):
+        return tuple(p for p in (self.mixer, self.mixer_post, self.feed_forward, self.feed_forward_post) if p is not None)
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return [s for p in self.parts() for s in p.tensor_specs()]
+
+    def bind(self, tensors, runtime) -> None:
+        for p in self.parts():
+            p.bind(tensors, runtime)
+
+    def linears(self) -> list:
+        return [lin for p in self.parts() for lin in p.linears()]
+
+    def cache_specs(self) -> list:
+        if hasattr(self.mixer, "cache_specs"):
+            return list(self.mixer.cache_specs())
+        spec = self.mixer.cache_spec()
+        return [] if spec is None else [spec]
+
+    def step_arrays(self) -> list:
+        return self.mixer.step_arrays()
+
+    @staticmethod
+    def _post(term: Partials, norm) -> Partials:
+        if term.outer is not None:
+            raise ValueError("a sublayer's result already carries a norm of its sum")
+        return Partials(term.data, term.bias, term.post, term.scale, term.more, PostNorm(norm.gain, norm.spec.eps, kind="rms"))
+
+    def forward(self, ctx, state: Hidden, caches: list) -> None:
+        from pyre_amd.hip import ops
+
+        h = ctx.workspace.get("block.h", (ctx.n_tokens, state.resid.shape[1]), ctx.dtype)
+        ops.add_rms_terms(state.resid, state.pending, None, 0.0, h)   # the pending term joins the stream; h = the stream
+        cache = caches if hasattr(self.mixer, "cache_specs") else (caches[0] if caches else None)
+        state.pending = self._post(self.mixer.forward(ctx, h, cache), self.mixer_post)
+        if self.feed_forward is None:
+            return
+        ops.add_rms_terms(state.resid, state.pending, None, 0.0, h)
+        state.pending = self._post(self.feed_forward.forward(ctx, h), self.feed_forward_post)

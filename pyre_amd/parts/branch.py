@@ -6,7 +6,7 @@ from __future__ import annotations
 
 import torch
 
-from pyre_amd.hip.ops import Partials
+from pyre_amd.hip.ops import Partials, PostNorm
 from pyre_amd.parts.base import Mixer, ParallelMixerSpec, TensorSpec, make_part, take
 from pyre_amd.parts.linear import Linear
 
@@ -46,6 +46,12 @@ class BranchMixer(Mixer):
     def attend(self, ctx, proj: Partials, col0: int, cache, o: torch.Tensor, scale: float) -> None:
         raise NotImplementedError
 
+    def cache_specs(self) -> list:
+        """What the mixer keeps, one description per cache (a mixer with pages and a state of its own has two);
+        ``attend`` gets the one view, or the list of them if there are several."""
+        spec = self.cache_spec()
+        return [] if spec is None else [spec]
+
     # ---- standing alone
     def tensor_specs(self) -> list[TensorSpec]:
         return [*self.in_tensors(), self.out_tensor(), *self.other_tensors()]
@@ -65,6 +71,8 @@ class BranchMixer(Mixer):
         n = ctx.n_tokens
         proj = self._in.forward(ctx, h, n)
         o = ctx.workspace.get(f"{self.role}.o", (n, self.inner), ctx.dtype)
+        if isinstance(cache, (list, tuple)) and len(self.cache_specs()) <= 1:  # a block that hands over all its views
+            cache = cache[0] if cache else None
         self.attend(ctx, proj, 0, cache, o, 1.0)
         return self._out.forward(ctx, o, n)
 
@@ -81,8 +89,12 @@ def _stacked(names, tensors, dim):
 
 class ParallelMixer(Mixer):
     """sum_i scale_i * branch_i(h). One input product for all branches, one output product over
-    [scale_0 o_0 | scale_1 o_1 | ...] against [Wo_0 | Wo_1 | ...]; every branch keeps its own cache
-    (``cache_specs``: one description per branch that keeps something, in their order)."""
+    [scale_0 o_0 | scale_1 o_1 | ...] against [Wo_0 | Wo_1 | ...]; every branch keeps its own caches
+    (``cache_specs``: the branches' descriptions in their order).
+
+    With ``out_norms`` every branch's result is normed over the hidden size before the sum, so the output products
+    stay apart (one per branch); none of the norms runs here: the results are handed on as pending terms, each with
+    its norm and factor, and the kernel that adds them to the residual stream applies both."""
 
     def __init__(self, spec: ParallelMixerSpec):
         if len(spec.branches) != len(spec.scales) or not spec.branches:
@@ -92,18 +104,23 @@ class ParallelMixer(Mixer):
         for b in self.branches:
             if not isinstance(b, BranchMixer):
                 raise ValueError(f"parallel mixer: {type(b).__name__} cannot share its products")
+        if spec.out_norms is not None and (len(spec.out_norms) != len(spec.branches) or len(spec.branches) > 2):
+            raise ValueError("parallel mixer: one output norm per branch, and at most two branches that are normed apart")
         self.inner = sum(b.inner for b in self.branches)
         self.proj = self.out = None   # made when the tensors are bound: a size may be the file's to say
+        self.outs: list[Linear] = []  # with out_norms: one output product per branch
+        self.out_gains: list[torch.Tensor] = []
         self.first_column: list[int] = []
 
     def cache_specs(self) -> list:
-        return [s for s in (b.cache_spec() for b in self.branches) if s is not None]
+        return [s for b in self.branches for s in b.cache_specs()]
 
     def step_arrays(self) -> list:
         return [a for b in self.branches for a in b.step_arrays()]
 
     def tensor_specs(self) -> list[TensorSpec]:
-        return [s for b in self.branches for s in (*b.in_tensors(), b.out_tensor(), *b.other_tensors())]
+        norms = [TensorSpec(n, (self.spec.hidden_size,), init="gain") for n in (self.spec.out_norms or ())]
+        return [s for b in self.branches for s in (*b.in_tensors(), b.out_tensor(), *b.other_tensors())] + norms
 
     def bind(self, tensors, runtime) -> None:
         # every branch's columns start at a multiple of eight (rows of zeros between them), so that the
@@ -121,24 +138,45 @@ class ParallelMixer(Mixer):
             parts += mine
             col += rows
         self.proj = Linear(self.spec.hidden_size, col, "mix.in")
-        self.out = Linear(self.inner, self.spec.hidden_size, "mix.out")
         self.proj.set(torch.cat(parts, dim=0))
         del parts, mine
-        self.out.set(_stacked([b.out_tensor().name for b in self.branches], tensors, 1))
+        if self.spec.out_norms is None:
+            self.out = Linear(self.inner, self.spec.hidden_size, "mix.out")
+            self.out.set(_stacked([b.out_tensor().name for b in self.branches], tensors, 1))
+        else:
+            for i, (b, name) in enumerate(zip(self.branches, self.spec.out_norms)):
+                lin = Linear(b.inner, self.spec.hidden_size, f"mix.out{i}")
+                lin.set(take(tensors, b.out_tensor().name))
+                self.outs.append(lin)
+                self.out_gains.append(take(tensors, name).contiguous())
         for b in self.branches:
             b.bind_others(tensors, runtime)
 
     def linears(self) -> list:
-        return [self.proj, self.out]
+        return [self.proj, *([self.out] if self.out is not None else self.outs)]
 
     def forward(self, ctx, h, caches):
         n = ctx.n_tokens
         proj = self.proj.forward(ctx, h, n)
-        o = ctx.workspace.get("mix.o", (n, self.inner), ctx.dtype)
+        apart = self.spec.out_norms is not None
+        o = None if apart else ctx.workspace.get("mix.o", (n, self.inner), ctx.dtype)
         views = iter(caches or [])
         at = 0
-        for b, scale, col in zip(self.branches, self.spec.scales, self.first_column):
-            cache = next(views) if b.cache_spec() is not None else None
-            b.attend(ctx, proj, col, cache, o[:, at:at + b.inner], float(scale))
-            at += b.inner
-        return self.out.forward(ctx, o, n)
+        terms = []
+        for i, (b, scale, col) in enumerate(zip(self.branches, self.spec.scales, self.first_column)):
+            mine = [next(views) for _ in b.cache_specs()]
+            cache = mine[0] if len(mine) == 1 else (mine or None)
+            if not apart:
+                b.attend(ctx, proj, col, cache, o[:, at:at + b.inner], float(scale))
+                at += b.inner
+                continue
+            # the branch's own rows, output product and norm; its factor rides on the pending term
+            rows = ctx.workspace.get(f"mix.o{i}", (n, b.inner), ctx.dtype)
+            b.attend(ctx, proj, col, cache, rows, 1.0)
+            p = self.outs[i].forward(ctx, rows, n)
+            terms.append(Partials(p.data, p.bias, PostNorm(self.out_gains[i], self.spec.norm_eps, kind="rms"), float(scale)))
+        if not apart:
+            return self.out.forward(ctx, o, n)
+        for first, second in zip(terms, terms[1:]):
+            first.more = second
+        return terms[0]

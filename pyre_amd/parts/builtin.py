@@ -2,16 +2,17 @@
 
 from pyre_amd.parts.attention import Attention
 from pyre_amd.parts.base import register_part
-from pyre_amd.parts.block import ParallelBlock, PreNormBlock, SandwichBlock
+from pyre_amd.parts.block import ParallelBlock, PostNormBlock, PreNormBlock, SandwichBlock
 from pyre_amd.parts.branch import ParallelMixer
 from pyre_amd.parts.capped_attention import CappedAttention
-from pyre_amd.parts.embedding import LMHead, TokenEmbedding
-from pyre_amd.parts.feedforward import ClippedGLU, GeluGLU, SwiGLU
+from pyre_amd.parts.embedding import BigramEmbedding, LMHead, TokenEmbedding
+from pyre_amd.parts.feedforward import ClippedGLU, GeluGLU, ReluSquaredMLP, SwiGLU
 from pyre_amd.parts.latent_attention import LatentAttention
-from pyre_amd.parts.linear_attention import GatedLinearAttention
-from pyre_amd.parts.moe import SigmoidMoE
+from pyre_amd.parts.linear_attention import GatedLinearAttention, Retention
+from pyre_amd.parts.moe import GroupedSoftmaxMoE, SigmoidMoE
 from pyre_amd.parts.norm import LayerNorm, RMSNorm, TanhNorm
 from pyre_amd.parts.rotary import NoPosition, RotaryEncoding
+from pyre_amd.parts.sink_attention import SinkAttention
 from pyre_amd.parts.tied_attention import TiedAttention
 
 register_part("mixer", "attention", Attention)
@@ -34,3 +35,9 @@ register_part("feed_forward", "gelu_glu", GeluGLU)
 register_part("feed_forward", "sigmoid_moe", SigmoidMoE)
 register_part("norm", "tanh_norm", TanhNorm)
 register_part("block", "parallel_block", ParallelBlock)
+register_part("embedding", "bigram_embedding", BigramEmbedding)
+register_part("block", "post_norm", PostNormBlock)
+register_part("mixer", "sink_attention", SinkAttention)
+register_part("mixer", "retention", Retention)
+register_part("feed_forward", "relu2_mlp", ReluSquaredMLP)
+register_part("feed_forward", "grouped_softmax_moe", GroupedSoftmaxMoE)

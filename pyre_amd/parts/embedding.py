@@ -5,7 +5,7 @@ from __future__ import annotations
 import torch
 
 from pyre_amd.hip import ops
-from pyre_amd.parts.base import EmbeddingSpec, LMHeadSpec, Part, TensorSpec
+from pyre_amd.parts.base import BigramEmbeddingSpec, EmbeddingSpec, LMHeadSpec, Part, StateCacheSpec, TensorSpec
 from pyre_amd.parts.linear import Linear
 
 
@@ -23,6 +23,37 @@ class TokenEmbedding(Part):
     def forward(self, ctx, resid: torch.Tensor) -> None:
         """resid[n] = float32(table[token n]): the residual stream starts here."""
         ops.embed(self.table, ctx.tokens, resid)
+
+
+class BigramEmbedding(Part):
+    """table[token] + pairs[row of (previous token, token)]: a second table indexed by a hash of the pair, whose last
+    row is for a request's first token. The previous token of the first token that a request brings in a step is state
+    that the request keeps on the device (one float32 whose value is the token's number, exact below 2^24), so a step
+    whose tokens are results still on the device needs nothing from the host."""
+
+    def __init__(self, spec: BigramEmbeddingSpec):
+        if spec.buckets <= 0 or spec.mul_prev < 0 or spec.mul_cur < 0:
+            raise ValueError("bigram embedding: buckets must be positive, the multipliers not negative")
+        if spec.vocab_size >= 1 << 24:
+            raise ValueError("bigram embedding: the previous token is kept as a float32, which holds numbers below 2^24")
+        self.spec = spec
+        self.table = self.pairs = None
+
+    def cache_specs(self) -> list:
+        return [StateCacheSpec((1,), "float32")]
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        s = self.spec
+        return [TensorSpec(s.name, (s.vocab_size, s.hidden_size)), TensorSpec(s.pairs_name, (s.buckets + 1, s.hidden_size))]
+
+    def bind(self, tensors, runtime) -> None:
+        self.table = tensors[self.spec.name].contiguous()
+        self.pairs = tensors[self.spec.pairs_name].to(self.table.dtype).contiguous()
+
+    def forward(self, ctx, resid: torch.Tensor, caches: list) -> None:
+        s = self.spec
+        ops.bigram_embed(self.table, self.pairs, ctx.tokens, ctx.positions, ctx.seq_of_token, ctx.q_start,
+                         caches[0].tensor, caches[0].slots, resid, s.buckets, s.mul_prev, s.mul_cur)
 
 
 class LMHead(Part):

@@ -91,7 +91,8 @@ def mid_ksplit(n_out: int, k: int, block_rows: int = 64, units: int = DEFAULT_UN
 # 0.026 of short portions, whose products hand on float32 partial sums anyway).
 LIBRARY_F32_ROLES = frozenset({"attn.qkv", "attn.out", "mix.in", "mix.out", "cattn.in", "cattn.out", "gla.in", "gla.out",
                                "glu.down", "tattn.qk", "tattn.out", "lattn.in", "lattn.out", "geglu.down", "moe.router",
-                               "moe.down"})
+                               "moe.down", "mix.out0", "mix.out1", "sattn.in", "sattn.out", "ret.in", "ret.out",
+                               "relu2.down", "gmoe.router", "gmoe.down"})
 
 
 def _is_bf16(ctx, lin, x) -> bool:

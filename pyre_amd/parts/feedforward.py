@@ -6,7 +6,7 @@ import torch
 
 from pyre_amd.hip import ops
 from pyre_amd.parts import fast
-from pyre_amd.parts.base import ClippedGLUSpec, FeedForward, GeluGLUSpec, SwiGLUSpec, TensorSpec, take
+from pyre_amd.parts.base import ClippedGLUSpec, FeedForward, GeluGLUSpec, ReluSquaredMLPSpec, SwiGLUSpec, TensorSpec, take
 from pyre_amd.parts.linear import Linear, linear_specs
 
 
@@ -117,4 +117,32 @@ class GeluGLU(FeedForward):
             gu = self.gate_up.forward(ctx, h, n)
             limit, slope, shift, cubic = self.UNIT
             ops.clipped_glu(gu, act, n, limit, slope, shift, cubic)
+        return self.down.forward(ctx, act, n)
+
+
+class ReluSquaredMLP(FeedForward):
+    """down(relu(up(x))^2): no gate, the activation is the square of the positive part."""
+
+    def __init__(self, spec: ReluSquaredMLPSpec):
+        self.spec = spec
+        self.up = Linear(spec.hidden_size, spec.intermediate_size, "relu2.up")
+        self.down = Linear(spec.intermediate_size, spec.hidden_size, "relu2.down")
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        s, p = self.spec, self.spec.prefix
+        return [TensorSpec(f"{p}.up", (s.intermediate_size, s.hidden_size)),
+                TensorSpec(f"{p}.down", (s.hidden_size, s.intermediate_size))]
+
+    def bind(self, tensors, runtime) -> None:
+        p = self.spec.prefix
+        self.up.set(take(tensors, f"{p}.up"))
+        self.down.set(take(tensors, f"{p}.down"))
+
+    def linears(self) -> list:
+        return [self.up, self.down]
+
+    def forward(self, ctx, h):
+        n = ctx.n_tokens
+        act = ctx.workspace.get("ffn.act", (n, self.spec.intermediate_size), ctx.dtype)
+        ops.relu2(self.up.forward(ctx, h, n), act, n)
         return self.down.forward(ctx, act, n)

@@ -53,7 +53,8 @@ class LayeredModel(Part):
 
     def cache_specs(self) -> list[list]:
         """What each entry of the order keeps: a list of cache descriptions, empty for an
-        entry that keeps nothing or reads another entry's caches."""
+        entry that keeps nothing or reads another entry's caches. An embedding that keeps state
+        has an entry of its own behind the last layer's."""
         out: list[list] = []
         for pos, call in enumerate(self.schedule):
             own = list(self.layers[call.layer].cache_specs())
@@ -65,6 +66,8 @@ class LayeredModel(Part):
                 raise ValueError(f"order entry {pos} reads the caches of entry {call.cache_from}, which keeps "
                                  f"{len(theirs)} of other kinds than the {len(own)} that this layer wants")
             out.append([])
+        if hasattr(self.embedding, "cache_specs"):  # an embedding with state of its own: one more entry, behind the layers'
+            out.append(list(self.embedding.cache_specs()))
         return out
 
     def tensor_uses(self) -> dict[str, int]:
@@ -90,7 +93,10 @@ class LayeredModel(Part):
         residual stream with the pending term added: a copy, made for the tap)."""
         n = ctx.n_tokens
         resid = ctx.workspace.get("resid", (n, self.spec.hidden_size), torch.float32)
-        self.embedding.forward(ctx, resid)
+        if hasattr(self.embedding, "cache_specs"):
+            self.embedding.forward(ctx, resid, caches[len(self.schedule)])
+        else:
+            self.embedding.forward(ctx, resid)
         state = Hidden(resid)
         for pos, call in enumerate(self.schedule):
             self.layers[call.layer].forward(ctx, state, caches[pos])
@@ -107,18 +113,26 @@ class LayeredModel(Part):
         """The residual stream as it stands after a layer, the term that the next norm would add
         included (its partial sums in their order, then the bias)."""
         rows = state.resid[:ctx.n_tokens].clone()
+
+        def normed(term, post):
+            if post is None:
+                return term
+            if post.kind == "rms":
+                term = term / torch.sqrt((term * term).mean(-1, keepdim=True) + post.eps) * post.gain.float()
+            else:
+                dev = term - term.mean(-1, keepdim=True)
+                term = dev / torch.sqrt((dev * dev).mean(-1, keepdim=True) + post.eps) * post.gain.float()
+            return term if post.scale is None else term * post.scale.float()
+
         p = state.pending
+        outer = p.outer if p is not None else None
+        total = torch.zeros_like(rows)
         while p is not None:
             term = torch.zeros_like(rows)
             for i in range(p.count):
                 term += p.data[i, :ctx.n_tokens].float()
             if p.bias is not None:
                 term += p.bias.float()
-            if p.post is not None:  # the term's own norm and scale, as the next norm's kernel applies them
-                dev = term - term.mean(-1, keepdim=True)
-                term = dev / torch.sqrt((dev * dev).mean(-1, keepdim=True) + p.post.eps) * p.post.gain.float()
-                if p.post.scale is not None:
-                    term = term * p.post.scale.float()
-            rows += term * p.scale
+            total += normed(term, p.post) * p.scale  # the term's own norm and scale, as the next norm's kernel applies them
             p = p.more
-        return rows
+        return rows + normed(total, outer)

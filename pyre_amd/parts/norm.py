@@ -12,12 +12,17 @@ class RMSNorm(Norm):
         self.gain = None
 
     def tensor_specs(self) -> list[TensorSpec]:
-        return [TensorSpec(f"{self.spec.prefix}.weight", (self.spec.hidden_size,), init="gain")]
+        return [TensorSpec(self.spec.tensor, (self.spec.hidden_size,), init="gain")]
 
     def bind(self, tensors, runtime) -> None:
-        self.gain = tensors[f"{self.spec.prefix}.weight"].contiguous()
+        self.gain = tensors[self.spec.tensor].contiguous()
 
     def forward(self, ctx, resid, delta, out, rows=None) -> None:
+        if delta is not None and (delta.post is not None or delta.more is not None or delta.outer is not None
+                                  or delta.scale != 1.0):
+            # a pending term that is normed or scaled before it is added, or comes with another
+            ops.add_rms_terms(resid, delta, self.gain, self.spec.eps, out, rows)
+            return
         ops.add_rmsnorm(resid, delta, self.gain, self.spec.eps, out, rows)
 
 
