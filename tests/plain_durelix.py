@@ -164,31 +164,46 @@ def dense_ff(h, w, p):
     return torch.relu(h @ w[f"{p}.up"].T) ** 2 @ w[f"{p}.down"].T
 
 
-def route(h, w, p, c):
+def choose(s, correction, top, count, keep):
+    """The experts chosen for one token with scores ``s``: by s + correction, among the experts of the ``keep`` of
+    ``count`` equal groups of neighbours whose largest such number is largest (the lower index among equals). Also
+    returns how close the call was: the least gap between something taken and the best thing left out."""
+    choice = s + correction
+    size = len(s) // count
+    tops = [float(choice[g * size:(g + 1) * size].max()) for g in range(count)]
+    best = sorted(range(count), key=lambda g: (-tops[g], g))
+    allowed = [e for g in best[:keep] for e in range(g * size, (g + 1) * size)]
+    ranked = sorted(allowed, key=lambda e: (-float(choice[e]), e))
+    gap = math.inf
+    if keep < count:
+        gap = min(gap, tops[best[keep - 1]] - tops[best[keep]])
+    if top < len(ranked):
+        gap = min(gap, float(choice[ranked[top - 1]] - choice[ranked[top]]))
+    return ranked[:top], gap
+
+
+def route(h, w, p, c, calls=None):
     """For every token the chosen experts and their weights, [(expert, weight), ...]: scores softmax(router h) over
-    experts and identity experts alike; the choice goes by score + correction among the experts of the ``keep``
-    groups (of neighbours) whose largest such number is largest; the weight is the score itself."""
+    experts and identity experts alike; the weight of a chosen expert is its score itself. ``calls`` collects, per
+    token, how close the choice was."""
     r = c["router"]
-    total = r["experts"] + r.get("identity", 0)
     groups = r.get("groups") or {"count": 1, "keep": 1}
-    size = total // groups["count"]
     out = []
     for t in range(h.shape[0]):
         s = torch.softmax(w[f"{p}.router"] @ h[t], -1)
-        choice = s + w[f"{p}.correction"]
-        best = sorted(range(groups["count"]), key=lambda g: (-float(choice[g * size:(g + 1) * size].max()), g))
-        allowed = [e for g in best[:groups["keep"]] for e in range(g * size, (g + 1) * size)]
-        chosen = sorted(allowed, key=lambda e: (-float(choice[e]), e))[:r["top"]]
+        chosen, gap = choose(s, w[f"{p}.correction"], r["top"], groups["count"], groups["keep"])
+        if calls is not None:
+            calls.append(gap)
         out.append([(e, s[e]) for e in chosen])
     return out
 
 
-def moe_ff(h, w, p, c):
+def moe_ff(h, w, p, c, calls=None):
     """The weighted sum of the chosen experts' results; an expert is down(silu(gate h) * (up h)), an identity
     expert (the last ``identity`` outputs of the router) hands the row back as it is."""
     real = c["router"]["experts"]
     out = torch.zeros_like(h)
-    for t, picks in enumerate(route(h, w, p, c)):
+    for t, picks in enumerate(route(h, w, p, c, calls)):
         for e, weight in picks:
             if e >= real:
                 out[t] += weight * h[t]
@@ -198,8 +213,12 @@ def moe_ff(h, w, p, c):
     return out
 
 
-def feed_forward(h, w, p, c):
-    return dense_ff(h, w, p) if c["kind"] == "dense" else moe_ff(h, w, p, c)
+def feed_forward(h, w, p, c, calls=None):
+    return dense_ff(h, w, p) if c["kind"] == "dense" else moe_ff(h, w, p, c, calls)
+
+
+#: layer type -> its mixer (h, w, prefix, the layer's 'mixer' entry, eps); tests of one branch alone add theirs
+MIXERS = {"parallel": parallel_mixer}
 
 
 # ----------------------------------------------------------------------------- the model
@@ -217,19 +236,31 @@ def embed(w, cfg, ids):
     return x
 
 
-def forward(w, cfg, ids, return_hidden=False):
-    """Logits [T, vocab] of one sequence (and the residual stream after every layer)."""
+def forward(w, cfg, ids, return_hidden=False, calls=None):
+    """Logits [T, vocab] of one sequence (and the residual stream after every layer). ``calls``: a list that
+    receives one list per routed layer, how close each token's choice of experts was."""
     eps = cfg["norm"]["eps"]
     x = embed(w, cfg, ids)
     hidden = []
     for n, layer in enumerate(cfg["layers"]):
         p = f"l{n}"
-        if layer["type"] != "parallel":
-            raise ValueError(f"layer type {layer['type']!r}")
         # every sublayer reads the stream itself; its result is normed before it is added
-        x = x + rms_norm(parallel_mixer(x, w, f"{p}.mix", layer["mixer"], eps), w[f"{p}.norm1"], eps)
+        x = x + rms_norm(MIXERS[layer["type"]](x, w, f"{p}.mix", layer["mixer"], eps), w[f"{p}.norm1"], eps)
         if layer.get("mlp") is not None:
-            x = x + rms_norm(feed_forward(x, w, f"{p}.mlp", layer["mlp"]), w[f"{p}.norm2"], eps)
+            mine = [] if calls is not None and layer["mlp"]["kind"] == "moe" else None
+            x = x + rms_norm(feed_forward(x, w, f"{p}.mlp", layer["mlp"], mine), w[f"{p}.norm2"], eps)
+            if mine is not None:
+                calls.append(mine)
         hidden.append(x)
     logits = rms_norm(x, w["final.norm"], eps) @ w["embed"].T
     return (logits, hidden) if return_hidden else logits
+
+
+def closest_call(w, cfg, ids):
+    """Per position the least gap, over the routed layers, by which the choice of experts was made (inf without any)."""
+    calls = []
+    forward(w, cfg, ids, calls=calls)
+    out = torch.full((len(ids),), math.inf, dtype=F)
+    for layer in calls:
+        out = torch.minimum(out, torch.tensor(layer, dtype=F))
+    return out
