@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--model qwen2.5-7b]
     python bench.py --workload serve [--model qwen2.5-1.5b] [--requests 256] [--max-batch 256]
-    python bench.py --workload designs [--shapes 1.5b,7b] [--layers 4] [--designs qwen2,mafurax,nurasun]
+    python bench.py --workload designs [--shapes 1.5b,7b] [--layers 4] [--designs qwen2,mafurax,nurasun,durelix]
 
 A step is one decode step of the scheduler: every running request gets one new
 token (plan, one engine step over the paged cache, greedy sampling, token fed
@@ -36,7 +36,10 @@ Nurasun design, whose layers alternate between attention with tied values over r
 (the same heads, half of each rotated) and latent attention (the same heads over a compressed row of 128
 elements, every second such layer reading the rows of the one before), and between the gated unit of the
 same width and a mixture of 8 experts of a quarter of that width, of which a token takes 2 beside a
-shared expert of half the width (so a token's feed-forward work is the dense one's). For each:
+shared expert of half the width (so a token's feed-forward work is the dense one's), and the Durelix design at
+the Mafurax design's split of the heads (a window of 1,024 tokens behind a convolution of four taps; layers alternate
+between down(relu(up)^2) of the same width and a mixture of 8 gated experts of a quarter of it and 2 identity experts).
+For each:
 the prefill of a 2,048-token prompt, decode steps at 8 and 64 requests with contexts of 4,096, and
 the device time of every kernel of a prefill step and of a decode step at 8 requests.
 
@@ -249,7 +252,22 @@ def designs(args) -> dict:
             nura.append(layer)
         nurasun = {"architecture": "Nurasun", "vocab": sh["vocab"], "width": sh["width"], "layers": nura, "norm": {"eps": 1e-6},
                    "residual_mult": 0.5, "logit_softcap": 30.0}
-        made = {"qwen2": qwen, "mafurax": mafurax, "nurasun": nurasun}
+        # Durelix at the Mafurax design's split of the heads: a window of 1,024 tokens behind a convolution of four taps,
+        # whole heads turned, decays from 1 - 2^-5 to 1 - 2^-10; layers alternate between the dense feed-forward and a
+        # mixture of 8 experts of a quarter of its width and 2 identity experts, in two groups of which a token's 2
+        # experts come from one
+        heads_r = sh["heads"] // 2
+        dleft = {"heads": sh["heads"] // 2, "kv_heads": max(1, sh["kv_heads"] // 2), "dim": sh["head"], "vdim": sh["head"],
+                 "scale": sh["head"] ** -0.5, "mask": {"size": 1024}, "conv": 4, "rot": {"base": 1e4, "dims": sh["head"]}}
+        dright = {"heads": heads_r, "dim": sh["head"], "vdim": sh["head"], "rot": {"base": 1e6, "dims": sh["head"]},
+                  "decay": [1.0 - 2.0 ** (-5.0 - 5.0 * i / max(1, heads_r - 1)) for i in range(heads_r)]}
+        dmix = {"kind": "moe", "expert": {"ff": sh["ff"] // 4},
+                "router": {"experts": 8, "identity": 2, "top": 2, "groups": {"count": 2, "keep": 1}}}
+        durelix = {"architecture": "Durelix", "vocab": sh["vocab"], "width": sh["width"], "norm": {"eps": 1e-6},
+                   "embedding": {"bigram": {"buckets": 65521, "mul_prev": 1000003, "mul_cur": 31}},
+                   "layers": [{"type": "parallel", "mixer": {"left": dleft, "right": dright},
+                               "mlp": dmix if i % 2 else {"kind": "dense", "ff": sh["ff"]}} for i in range(layers)]}
+        made = {"qwen2": qwen, "mafurax": mafurax, "nurasun": nurasun, "durelix": durelix}
         return {name: config_from_dict(made[name]) for name in args.designs.split(",") if name}
 
     def kernels_of(run, per: int) -> dict:
@@ -398,7 +416,8 @@ def main() -> int:
     ap.add_argument("--model", default=None, help="preset shape (qwen2.5-7b; for --workload serve qwen2.5-1.5b)")
     ap.add_argument("--workload", default="decode", choices=["decode", "serve", "designs"])
     ap.add_argument("--shapes", default="1.5b,7b", help="designs: the layer sizes to compare at (1.5b, 7b)")
-    ap.add_argument("--designs", default="qwen2,mafurax,nurasun", help="designs: which of qwen2, mafurax, nurasun to measure")
+    ap.add_argument("--designs", default="qwen2,mafurax,nurasun,durelix",
+                    help="designs: which of qwen2, mafurax, nurasun, durelix to measure")
     ap.add_argument("--requests", type=int, default=256, help="serve: number of requests")
     ap.add_argument("--max-batch", type=int, default=256, help="serve: requests that run at a time")
     ap.add_argument("--seed", type=int, default=0, help="serve: seed of the lengths and token ids")

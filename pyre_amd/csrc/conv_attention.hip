@@ -3,7 +3,8 @@
 //
 //   u_t      = the product's columns of token t (sum of its partial sums): nq query heads and nkv key heads of dk,
 //              nkv value heads of dv, then nq * dv gate columns
-//   y_t[c]   = sum_j taps[c][j] * u_(t - (T - 1) + j)[c],  j = 0 .. T - 1, for the query, key and value channels c;
+//   y_t[c]   = sum_j taps[j][c] * u_(t - (T - 1) + j)[c],  j = 0 .. T - 1, for the query, key and value channels c
+//              (the taps as float32 [T][channels]: a tap's weights of neighbouring channels lie together);
 //              rows before the request's first token are zero, rows before the step's first token of the request come
 //              from the request's state, which holds its last T - 1 rows u (float32 [T - 1][channels], oldest first)
 //   q, k     = per head: y / sqrt(mean(y^2) + eps) * gain   (gains over dk, shared by the heads; or not normed)
@@ -20,6 +21,7 @@
 // depend on where a step begins. All arithmetic float32.
 #include "pyre_api.h"
 #include "pyre_common.h"
+#include "pyre_vec4.h"
 
 using namespace pyre;
 
@@ -34,7 +36,7 @@ struct ConvIn {
   int proj_dt, n_partials;
   size_t partial_stride;
   int ld, col0;
-  const float* taps_w;   // [channels][taps] or null
+  const float* taps_w;   // [taps][channels] or null
   int taps;
   const float* state;    // [slots][taps - 1][channels] or null
   int channels;
@@ -51,14 +53,13 @@ __device__ inline float product_value(const ConvIn& in, int n, int col) {
 // Channel `ch` of token n after the convolution; `run` is the token's index among its request's tokens of the step.
 __device__ inline float conv_value(const ConvIn& in, int n, int run, int slot, int ch) {
   if (!in.taps_w) return product_value(in, n, ch);
-  const float* w = in.taps_w + static_cast<size_t>(ch) * in.taps;
   float y = 0.f;
   for (int j = 0; j < in.taps; ++j) {
     const int back = in.taps - 1 - j;  // this tap's input lies `back` tokens before n
     float u;
     if (run - back >= 0) u = product_value(in, n - back, ch);
     else u = in.state[(static_cast<size_t>(slot) * (in.taps - 1) + (in.taps - 1 + run - back)) * in.channels + ch];
-    y = fmaf(w[j], u, y);
+    y = fmaf(in.taps_w[static_cast<size_t>(j) * in.channels + ch], u, y);
   }
   return y;
 }
@@ -125,6 +126,100 @@ __global__ __launch_bounds__(kThreads) void conv_qkv_write_kernel(
       gate_out[static_cast<size_t>(n) * nq * dv + i] = 1.f / (1.f + expf(-product_value(in, n, in.channels + i)));
 }
 
+
+// The same with a wave per block, four elements a lane and an element's partial sums asked for together: blocks
+// 0 .. nq + nkv - 1 of a token take a head each, the blocks behind them 256 value or gate columns each. Head sizes, the
+// product's width, first column and stride are multiples of four; queries and caches share one element type. The sums
+// run in the order of the kernel above: the same bits.
+constexpr int kVecTaps = 8;  // the most taps of this form
+template <typename TP>
+__device__ inline float4 conv_value4(const ConvIn& in, const TP* proj, int n, int run, int slot, int ch) {
+  const TP* row = proj + static_cast<size_t>(n) * in.ld + in.col0 + ch;
+  if (!in.taps_w) return sum_partials4(row, in.partial_stride, in.n_partials);
+  float4 u[kVecTaps];
+#pragma unroll
+  for (int j = 0; j < kVecTaps; ++j) {  // every tap's input asked for before the first is used
+    if (j >= in.taps) break;
+    const int back = in.taps - 1 - j;
+    if (run - back >= 0) u[j] = sum_partials4(row - static_cast<size_t>(back) * in.ld, in.partial_stride, in.n_partials);
+    else u[j] = *reinterpret_cast<const float4*>(in.state + (static_cast<size_t>(slot) * (in.taps - 1) + (in.taps - 1 + run - back)) * in.channels + ch);
+  }
+  float4 y = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < kVecTaps; ++j) {
+    if (j >= in.taps) break;
+    const float4 w = *reinterpret_cast<const float4*>(in.taps_w + static_cast<size_t>(j) * in.channels + ch);
+    y = float4{fmaf(w.x, u[j].x, y.x), fmaf(w.y, u[j].y, y.y), fmaf(w.z, u[j].z, y.z), fmaf(w.w, u[j].w, y.w)};
+  }
+  return y;
+}
+
+template <typename TP, typename TC>
+__global__ __launch_bounds__(kWave) void conv_qkv_write_vec_kernel(
+    ConvIn in, const int* __restrict__ state_slots, const int* __restrict__ seq_of_token, const int* __restrict__ q_start,
+    const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps, const float* __restrict__ cos,
+    const float* __restrict__ sin, int rot, int neighbours, const int* __restrict__ positions, TC* __restrict__ q_out,
+    TC* __restrict__ k_cache, TC* __restrict__ v_cache, float* __restrict__ gate_out, const int* __restrict__ slots,
+    int nq, int nkv, int dk, int dv, int page_size, int write_kv) {
+  __shared__ __attribute__((aligned(16))) float xs[kMaxHead];
+  const int n = blockIdx.x, lane = threadIdx.x;
+  const int seq = seq_of_token[n], run = n - q_start[seq], st = state_slots[seq];
+  const int slot = write_kv ? slots[n] : -1;
+  const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+  const TP* proj = static_cast<const TP*>(in.proj);
+  if (static_cast<int>(blockIdx.y) >= nq + nkv) {
+    // 256 columns of the values, then of the gates
+    const int i = (static_cast<int>(blockIdx.y) - nq - nkv) * 4 * kWave + 4 * lane, nv = nkv * dv;
+    if (i < nv) {
+      if (slot >= 0) {
+        const int g = i / dv, e = i % dv;
+        Vec4<TC>::store(v_cache + ((static_cast<size_t>(page) * nkv + g) * page_size + off) * dv + e,
+                        conv_value4(in, proj, n, run, st, (nq + nkv) * dk + i));
+      }
+    } else if (gate_out && i - nv < nq * dv) {
+      const float4 z = sum_partials4(proj + static_cast<size_t>(n) * in.ld + in.col0 + in.channels + (i - nv), in.partial_stride, in.n_partials);
+      *reinterpret_cast<float4*>(gate_out + static_cast<size_t>(n) * nq * dv + (i - nv)) =
+          float4{1.f / (1.f + expf(-z.x)), 1.f / (1.f + expf(-z.y)), 1.f / (1.f + expf(-z.z)), 1.f / (1.f + expf(-z.w))};
+    }
+    return;
+  }
+  const int head = blockIdx.y, e = 4 * lane, half = rot / 2;
+  const bool mine = e < dk;
+  float4 x = {0.f, 0.f, 0.f, 0.f};
+  if (mine) x = conv_value4(in, proj, n, run, st, head * dk + e);
+  const float* gain = head < nq ? q_gain : k_gain;
+  if (gain) {
+    // the sum of squares in the order of the kernel above: a lane's elements e, e + 64, .. there, four neighbours here;
+    // both are wave sums of per-lane sums, a difference of rounding
+    const float inv = 1.f / sqrtf(wave_sum((x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w)) / static_cast<float>(dk) + eps);
+    if (mine) {
+      const float4 g = *reinterpret_cast<const float4*>(gain + e);
+      x = float4{x.x * inv * g.x, x.y * inv * g.y, x.z * inv * g.z, x.w * inv * g.w};
+    }
+  }
+  if (mine) *reinterpret_cast<float4*>(xs + e) = x;
+  __syncthreads();
+  if (!mine) return;
+  float y[4] = {x.x, x.y, x.z, x.w};
+  const size_t trig = static_cast<size_t>(positions[n]) * half;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int el = e + u;
+    if (el >= rot) continue;
+    // the pair's index, and whether this element is its first or its second
+    const int pair = neighbours ? el >> 1 : (el < half ? el : el - half);
+    const bool first = neighbours ? !(el & 1) : el < half;
+    const int partner = neighbours ? el ^ 1 : (first ? el + half : el - half);
+    float a, b;
+    if (first) rotate_pair(y[u], xs[partner], cos[trig + pair], sin[trig + pair], a, b);
+    else rotate_pair(xs[partner], y[u], cos[trig + pair], sin[trig + pair], a, b);
+    y[u] = first ? a : b;
+  }
+  const float4 out = {y[0], y[1], y[2], y[3]};
+  if (head < nq) Vec4<TC>::store(q_out + (static_cast<size_t>(n) * nq + head) * dk + e, out);
+  else if (slot >= 0) Vec4<TC>::store(k_cache + ((static_cast<size_t>(page) * nkv + (head - nq)) * page_size + off) * dk + e, out);
+}
+
 // A thread a channel, the rows of the new state in ascending order: row i takes the step's row len - (T - 1) + i of the
 // request or, where the step is shorter than that, the old state's row i + len, which lies further on and is still old.
 __global__ __launch_bounds__(kThreads) void conv_state_update_kernel(ConvIn in, float* __restrict__ state,
@@ -162,11 +257,23 @@ extern "C" int pyre_conv_qkv_write(const void* proj, int proj_dt, int n_partials
   if (n <= 0) return 0;
   const ConvIn in{proj, proj_dt, n_partials, static_cast<size_t>(partial_stride), ld, col0, taps_w, taps, conv_state,
                   (nq + nkv) * dk + nkv * dv};
-  PYRE_DISPATCH(cache_dt, TC,
-      hipLaunchKernelGGL(conv_qkv_write_kernel<TC>, dim3(n), dim3(kThreads), 0, stream, in, state_slots, seq_of_token,
-                         q_start, q_gain, k_gain, eps, cos, sin, rot, neighbours, positions, q_out, q_dt,
-                         static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), gate_out, slots, nq, nkv, dk, dv, page_size,
-                         write_kv));
+  const auto a16 = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+  const int tail_blocks = (nkv * dv + (gate_out ? nq * dv : 0) + 4 * kWave - 1) / (4 * kWave);
+  if (taps <= kVecTaps && dk % 4 == 0 && dv % 4 == 0 && ld % 4 == 0 && col0 % 4 == 0 && partial_stride % 4 == 0 && q_dt == cache_dt &&
+      nq + nkv + tail_blocks <= 65535 && a16(proj) && a16(q_out) && a16(k_cache) && a16(v_cache) && a16(gate_out) &&
+      a16(taps_w) && a16(conv_state) && a16(q_gain) && a16(k_gain)) {
+    PYRE_DISPATCH(proj_dt, TP, PYRE_DISPATCH(cache_dt, TC,
+        hipLaunchKernelGGL((conv_qkv_write_vec_kernel<TP, TC>), dim3(n, nq + nkv + tail_blocks), dim3(kWave), 0, stream, in,
+                           state_slots, seq_of_token, q_start, q_gain, k_gain, eps, cos, sin, rot, neighbours, positions,
+                           static_cast<TC*>(q_out), static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), gate_out, slots,
+                           nq, nkv, dk, dv, page_size, write_kv)));
+  } else {
+    PYRE_DISPATCH(cache_dt, TC,
+        hipLaunchKernelGGL(conv_qkv_write_kernel<TC>, dim3(n), dim3(kThreads), 0, stream, in, state_slots, seq_of_token,
+                           q_start, q_gain, k_gain, eps, cos, sin, rot, neighbours, positions, q_out, q_dt,
+                           static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), gate_out, slots, nq, nkv, dk, dv,
+                           page_size, write_kv));
+  }
   if (check_launch("conv_qkv_write")) return 1;
   if (taps > 1 && n_seqs > 0) {
     const int cols = (in.channels + kThreads - 1) / kThreads;

@@ -369,6 +369,58 @@ __global__ __launch_bounds__(kThreads) void retention_prepare_kernel(
   for (int i = tid; i < 2 * hv; i += kThreads) xr[3 * hk + i] = value(2 * hk + i);
 }
 
+// The same with a wave per block and four columns a lane: blocks 0 .. 2 heads - 1 of a token take a query or key head
+// each (the partners of a rotation exchanged through LDS), the blocks behind them 256 columns of [ld | v | g] each. The
+// head sizes, the product's width, first column and stride are multiples of four.
+template <typename TP>
+__global__ __launch_bounds__(kWave) void retention_prepare_vec_kernel(
+    const TP* __restrict__ proj, int n_partials, size_t partial_stride, int ld, int col0,
+    const float* __restrict__ log_decay, const float* __restrict__ cos, const float* __restrict__ sin, int rot,
+    int neighbours, const int* __restrict__ positions, float kscale, float* __restrict__ x, int heads, int dk, int dv) {
+  __shared__ __attribute__((aligned(16))) float xs[256];
+  const int n = blockIdx.x, lane = threadIdx.x;
+  const TP* in = proj + static_cast<size_t>(n) * ld + col0;
+  const int hk = heads * dk, hv = heads * dv, width = 3 * hk + 2 * hv, half = rot / 2;
+  float* xr = x + static_cast<size_t>(n) * width;
+  if (static_cast<int>(blockIdx.y) >= 2 * heads) {
+    const int i = (static_cast<int>(blockIdx.y) - 2 * heads) * 4 * kWave + 4 * lane;  // a column of [ld | v | g]
+    if (i < hk) {
+      const float l = log_decay[i / dk];  // four neighbours share a head: dk is a multiple of four
+      *reinterpret_cast<float4*>(xr + 2 * hk + i) = float4{l, l, l, l};
+    } else if (i < hk + 2 * hv) {
+      *reinterpret_cast<float4*>(xr + 2 * hk + i) = sum_partials4(in + 2 * hk + (i - hk), partial_stride, n_partials);
+    }
+    return;
+  }
+  const int head = blockIdx.y, e = 4 * lane;  // head counts query heads, then key heads
+  const bool mine = e < dk;
+  float4 v = {0.f, 0.f, 0.f, 0.f};
+  if (mine) {
+    v = sum_partials4(in + head * dk + e, partial_stride, n_partials);
+    *reinterpret_cast<float4*>(xs + e) = v;
+  }
+  __syncthreads();
+  if (!mine) return;
+  float y[4] = {v.x, v.y, v.z, v.w};
+  const size_t trig = static_cast<size_t>(positions[n]) * half;
+  const float f = head >= heads ? kscale : 1.f;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int el = e + u;
+    if (el < rot) {
+      const int pair = neighbours ? el >> 1 : (el < half ? el : el - half);
+      const bool first = neighbours ? !(el & 1) : el < half;
+      const int partner = neighbours ? el ^ 1 : (first ? el + half : el - half);
+      float a, b;
+      if (first) rotate_pair(y[u], xs[partner], cos[trig + pair], sin[trig + pair], a, b);
+      else rotate_pair(xs[partner], y[u], cos[trig + pair], sin[trig + pair], a, b);
+      y[u] = first ? a : b;
+    }
+    y[u] *= f;
+  }
+  *reinterpret_cast<float4*>(xr + head * dk + e) = float4{y[0], y[1], y[2], y[3]};
+}
+
 }  // namespace
 
 extern "C" int pyre_gla_prepare(const void* proj, int proj_dt, int n_partials, long partial_stride, int ld, int col0,
@@ -463,6 +515,15 @@ extern "C" int pyre_retention_prepare(const void* proj, int proj_dt, int n_parti
   PYRE_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= dk && (rot == 0 || (cos && sin)),
                "retention_prepare: %d turned elements of a head of %d need tables and an even number", rot, dk);
   if (n <= 0) return 0;
+  const int tail_blocks = (heads * dk + 2 * heads * dv + 4 * kWave - 1) / (4 * kWave);
+  if (dk % 4 == 0 && dv % 4 == 0 && dk <= 256 && ld % 4 == 0 && col0 % 4 == 0 && partial_stride % 4 == 0 &&
+      2 * heads + tail_blocks <= 65535 && reinterpret_cast<uintptr_t>(proj) % 16 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+    PYRE_DISPATCH(proj_dt, TP,
+        hipLaunchKernelGGL(retention_prepare_vec_kernel<TP>, dim3(n, 2 * heads + tail_blocks), dim3(kWave), 0, stream,
+                           static_cast<const TP*>(proj), n_partials, static_cast<size_t>(partial_stride), ld, col0,
+                           log_decay, cos, sin, rot, neighbours, positions, kscale, x, heads, dk, dv));
+    return check_launch("retention_prepare");
+  }
   hipLaunchKernelGGL(retention_prepare_kernel, dim3(n), dim3(kThreads), 0, stream, proj, proj_dt, n_partials,
                      static_cast<size_t>(partial_stride), ld, col0, log_decay, cos, sin, rot, neighbours, positions, kscale,
                      x, heads, dk, dv);

@@ -1245,7 +1245,7 @@ def conv_qkv_write(proj: Partials, col0: int, taps_w: torch.Tensor | None, conv_
                    slots: torch.Tensor | None, n: int, nq: int, nkv: int, dk: int, dv: int, page_size: int) -> None:
     """Finish a step's input product from column ``col0`` on (``nq`` query and ``nkv`` key heads of ``dk``, ``nkv`` value
     heads of ``dv``, then ``nq * dv`` gate columns if ``gate_out`` is given). Queries, keys and values first go through a
-    causal convolution over the request's tokens, ``taps_w`` float32 [channels, taps] (None: none), whose inputs before
+    causal convolution over the request's tokens, ``taps_w`` float32 [taps, channels] (None: none), whose inputs before
     the step's first token come from ``conv_state`` (float32 [slots, taps - 1, channels], the request's last projected
     rows; it is brought up to date after every token has read it). Then queries and keys are divided by their root mean
     square per head, times ``q_gain`` / ``k_gain`` over ``dk`` (None: not normed), and their first ``rot`` elements turned
@@ -1261,10 +1261,10 @@ def conv_qkv_write(proj: Partials, col0: int, taps_w: torch.Tensor | None, conv_
     _i32("q_start", q_start, n_seqs + 1), _i32("state_slots", state_slots, n_seqs)
     taps = 0
     if taps_w is not None:
-        taps = taps_w.shape[1]
-        if taps_w.dtype != torch.float32 or not taps_w.is_contiguous() or tuple(taps_w.shape) != (channels, taps) or \
+        taps = taps_w.shape[0]
+        if taps_w.dtype != torch.float32 or not taps_w.is_contiguous() or tuple(taps_w.shape) != (taps, channels) or \
                 not (1 <= taps <= CONV_MAX_TAPS):
-            raise KernelError(f"conv_qkv_write: the taps are contiguous float32 [{channels}, 1..{CONV_MAX_TAPS}]")
+            raise KernelError(f"conv_qkv_write: the taps are contiguous float32 [1..{CONV_MAX_TAPS}, {channels}]")
         if taps > 1:
             if conv_state is None or conv_state.dtype != torch.float32 or not conv_state.is_contiguous() or \
                     tuple(conv_state.shape[1:]) != (taps - 1, channels):

@@ -34,6 +34,8 @@ class BigramEmbedding(Part):
     def __init__(self, spec: BigramEmbeddingSpec):
         if spec.buckets <= 0 or spec.mul_prev < 0 or spec.mul_cur < 0:
             raise ValueError("bigram embedding: buckets must be positive, the multipliers not negative")
+        if spec.buckets >= 1 << 31:
+            raise ValueError("bigram embedding: more buckets than a 32-bit row number holds")
         if spec.vocab_size >= 1 << 24:
             raise ValueError("bigram embedding: the previous token is kept as a float32, which holds numbers below 2^24")
         self.spec = spec
@@ -52,8 +54,9 @@ class BigramEmbedding(Part):
 
     def forward(self, ctx, resid: torch.Tensor, caches: list) -> None:
         s = self.spec
+        # (p a + t b) mod m = (p (a mod m) + t (b mod m)) mod m: the kernel's 64-bit products hold whatever the multipliers are
         ops.bigram_embed(self.table, self.pairs, ctx.tokens, ctx.positions, ctx.seq_of_token, ctx.q_start,
-                         caches[0].tensor, caches[0].slots, resid, s.buckets, s.mul_prev, s.mul_cur)
+                         caches[0].tensor, caches[0].slots, resid, s.buckets, s.mul_prev % s.buckets, s.mul_cur % s.buckets)
 
 
 class LMHead(Part):

@@ -81,7 +81,8 @@ class SinkAttention(BranchMixer):
     def bind_others(self, tensors, runtime) -> None:
         s, p = self.spec, self.spec.prefix
         if s.conv_taps:
-            self.taps = torch.cat([take(tensors, f"{p}.{x}.conv").float() for x in ("q", "k", "v")], dim=0).contiguous()
+            # [taps, channels]: a tap's weights of neighbouring channels lie together
+            self.taps = torch.cat([take(tensors, f"{p}.{x}.conv").float() for x in ("q", "k", "v")], dim=0).t().contiguous()
         if s.qk_norm:
             self.q_gain = take(tensors, f"{p}.q.norm").float().contiguous()
             self.k_gain = take(tensors, f"{p}.k.norm").float().contiguous()
