@@ -38,7 +38,7 @@ elements, every second such layer reading the rows of the one before), and betwe
 same width and a mixture of 8 experts of a quarter of that width, of which a token takes 2 beside a
 shared expert of half the width (so a token's feed-forward work is the dense one's), and the Durelix design at
 the Mafurax design's split of the heads (a window of 1,024 tokens behind a convolution of four taps; layers alternate
-between down(relu(up)^2) of the same width and a mixture of 8 gated experts of a quarter of it and 2 identity experts).
+between down(relu(up)^2) of the same width and a mixture of 8 gated experts of a quarter of it and 4 identity experts).
 For each:
 the prefill of a 2,048-token prompt, decode steps at 8 and 64 requests with contexts of 4,096, and
 the device time of every kernel of a prefill step and of a decode step at 8 requests.
@@ -253,16 +253,16 @@ def designs(args) -> dict:
         nurasun = {"architecture": "Nurasun", "vocab": sh["vocab"], "width": sh["width"], "layers": nura, "norm": {"eps": 1e-6},
                    "residual_mult": 0.5, "logit_softcap": 30.0}
         # Durelix at the Mafurax design's split of the heads: a window of 1,024 tokens behind a convolution of four taps,
-        # whole heads turned, decays from 1 - 2^-5 to 1 - 2^-10; layers alternate between the dense feed-forward and a
-        # mixture of 8 experts of a quarter of its width and 2 identity experts, in two groups of which a token's 2
-        # experts come from one
+        # whole heads turned, decays from 0.9 to 0.9999; layers alternate between the dense feed-forward and a
+        # mixture of 8 experts of a quarter of its width and 4 identity experts, in three groups of which a token's 2
+        # experts come from the best two
         heads_r = sh["heads"] // 2
         dleft = {"heads": sh["heads"] // 2, "kv_heads": max(1, sh["kv_heads"] // 2), "dim": sh["head"], "vdim": sh["head"],
                  "scale": sh["head"] ** -0.5, "mask": {"size": 1024}, "conv": 4, "rot": {"base": 1e4, "dims": sh["head"]}}
         dright = {"heads": heads_r, "dim": sh["head"], "vdim": sh["head"], "rot": {"base": 1e6, "dims": sh["head"]},
-                  "decay": [1.0 - 2.0 ** (-5.0 - 5.0 * i / max(1, heads_r - 1)) for i in range(heads_r)]}
+                  "decay": [0.9 + 0.0999 * i / max(1, heads_r - 1) for i in range(heads_r)]}
         dmix = {"kind": "moe", "expert": {"ff": sh["ff"] // 4},
-                "router": {"experts": 8, "identity": 2, "top": 2, "groups": {"count": 2, "keep": 1}}}
+                "router": {"experts": 8, "identity": 4, "top": 2, "groups": {"count": 3, "keep": 2}}}
         durelix = {"architecture": "Durelix", "vocab": sh["vocab"], "width": sh["width"], "norm": {"eps": 1e-6},
                    "embedding": {"bigram": {"buckets": 65521, "mul_prev": 1000003, "mul_cur": 31}},
                    "layers": [{"type": "parallel", "mixer": {"left": dleft, "right": dright},

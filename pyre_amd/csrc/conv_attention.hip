@@ -11,9 +11,10 @@
 //   q, k     = their first `rot` elements turned by position: pairs (e, e + rot/2) or neighbours (2e, 2e + 1)
 //   gate     = sigmoid(u_t[gate columns])                   (float32, one per element of the heads' outputs)
 //
-// conv_qkv_write       one block a token: a wave takes a head at a time (four elements a lane, dk <= 256), norms it,
-//                      leaves it in LDS, turns the pairs and stores queries (rows) and keys (pages); values and gates
-//                      are dealt to all threads.
+// conv_qkv_write       a wave per token and head (four neighbouring elements a lane, dk <= 256): it norms the head,
+//                      leaves it in LDS, turns the pairs and stores queries (rows) and keys (pages); further waves take
+//                      256 columns of values and gates each. A form for any sizes and element types has one block a
+//                      token, whose waves take a head at a time.
 // conv_state_update    one block a request, after every token has read the old state: the last T - 1 rows u of the
 //                      request, taken from the step's rows and, for a step shorter than that, from the old state.
 //

@@ -64,11 +64,11 @@ ONES = model(31, 20, [
     layer(left(1, 1, 6, 3, 1.1, window=1, conv=1, rot=(7.0, 2)), right(1, 4, 5, (0.8,), rot=(3.0, 4)), moe(1, 1, 7)),
 ], eps=1e-3, bigram=(1, 1, 1))
 
-#: eight query heads on two groups, key heads beyond 128 elements, a router of two groups of which one is kept, no
+#: eight query heads on two groups, key heads beyond 128 elements, a router of three groups of which one is kept, no
 #: second embedding table
 WIDE = model(64, 64, [
-    layer(left(8, 2, 32, 32, 0.3, window=33, conv=4, rot=(20000.0, 32)), right(2, 32, 96, (0.95, 0.999), rot=(1e6, 16)),
-          moe(7, 3, 24, identity=1, groups=(2, 1))),
+    layer(left(8, 2, 32, 32, 0.3, window=33, conv=4, rot=(30000.0, 32)), right(2, 32, 96, (0.95, 0.999), rot=(2e5, 16)),
+          moe(9, 4, 24, identity=3, groups=(3, 1))),
     layer(left(2, 2, 136, 20, 0.1, window=18, conv=4, rot=(1000.0, 64)), right(2, 130, 16, (0.9, 0.99), rot=(100.0, 130)),
           dense(64)),
 ], eps=1e-6)
