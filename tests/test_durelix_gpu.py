@@ -358,7 +358,9 @@ def test_each_mixer_alone(kind, tmp_path):
     from pyre_amd.registry import register_architecture, unregister_architecture
     from pyre_amd.weights import write_random_model
 
-    mixers = {"left": [M.left(4, 2, 24, 16, 0.5, window=20, conv=3, rot=(100.0, 10)), M.left(5, 1, 7, 9, 0.8)],
+    # (nine taps: more than the kernel with four elements a lane takes, and more than the first portions are long)
+    mixers = {"left": [M.left(4, 2, 24, 16, 0.5, window=20, conv=3, rot=(100.0, 10)), M.left(5, 1, 7, 9, 0.8),
+                       M.left(2, 1, 12, 8, 0.6, window=5, conv=9, rot=(10.0, 4))],
               "right": [M.right(2, 16, 24, (0.9, 0.99), rot=(30.0, 16)), M.right(3, 33, 7, (1.0, 0.3, 0.97))]}[kind]
     raw = {"architectures": ["ToyOneBranch"], "vocab": 71, "width": 40, "norm": {"eps": 1e-5},
            "layers": [{"type": kind, "mixer": m, "mlp": None} for m in mixers]}
@@ -372,7 +374,8 @@ def test_each_mixer_alone(kind, tmp_path):
         want = {r: plain_rows(cfg, w, ids) for r, ids in reqs.items()}
         eng = engine_of(tmp_path, "float32")
         kinds = [[type(s).__name__ for s in c] for c in eng.model.cache_specs()]
-        assert kinds == ([["PagedCacheSpec", "StateCacheSpec"], ["PagedCacheSpec"]] if kind == "left" else [["StateCacheSpec"]] * 2)
+        assert kinds == ([["PagedCacheSpec", "StateCacheSpec"], ["PagedCacheSpec"], ["PagedCacheSpec", "StateCacheSpec"]]
+                         if kind == "left" else [["StateCacheSpec"]] * 2)
         assert_close(replay(eng, whole(reqs)), want, TOL["float32"])
         assert_close(replay(eng, in_portions(reqs, [5, 2, 30])), want, TOL["float32"])
         assert_close(replay(eng, one_by_one(reqs, 4)), want, TOL["float32"])
