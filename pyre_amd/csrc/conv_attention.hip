@@ -22,48 +22,16 @@
 // depend on where a step begins. All arithmetic float32.
 #include "pyre_api.h"
 #include "pyre_common.h"
+#include "pyre_conv.h"
 #include "pyre_vec4.h"
 
 using namespace pyre;
 
 namespace {
 
-constexpr int kThreads = 256;
+constexpr int kThreads = kConvThreads;
 constexpr int kMaxHead = 256;
 constexpr int kMaxTaps = 16;
-
-struct ConvIn {
-  const void* proj;
-  int proj_dt, n_partials;
-  size_t partial_stride;
-  int ld, col0;
-  const float* taps_w;   // [taps][channels] or null
-  int taps;
-  const float* state;    // [slots][taps - 1][channels] or null
-  int channels;
-};
-
-// Column `col` of the step's row `n` of the product.
-__device__ inline float product_value(const ConvIn& in, int n, int col) {
-  const size_t at = static_cast<size_t>(n) * in.ld + in.col0 + col;
-  float v = 0.f;
-  for (int p = 0; p < in.n_partials; ++p) v += load_as_float(in.proj, in.proj_dt, p * in.partial_stride + at);
-  return v;
-}
-
-// Channel `ch` of token n after the convolution; `run` is the token's index among its request's tokens of the step.
-__device__ inline float conv_value(const ConvIn& in, int n, int run, int slot, int ch) {
-  if (!in.taps_w) return product_value(in, n, ch);
-  float y = 0.f;
-  for (int j = 0; j < in.taps; ++j) {
-    const int back = in.taps - 1 - j;  // this tap's input lies `back` tokens before n
-    float u;
-    if (run - back >= 0) u = product_value(in, n - back, ch);
-    else u = in.state[(static_cast<size_t>(slot) * (in.taps - 1) + (in.taps - 1 + run - back)) * in.channels + ch];
-    y = fmaf(in.taps_w[static_cast<size_t>(j) * in.channels + ch], u, y);
-  }
-  return y;
-}
 
 template <typename TC>
 __global__ __launch_bounds__(kThreads) void conv_qkv_write_kernel(
@@ -219,21 +187,6 @@ __global__ __launch_bounds__(kWave) void conv_qkv_write_vec_kernel(
   const float4 out = {y[0], y[1], y[2], y[3]};
   if (head < nq) Vec4<TC>::store(q_out + (static_cast<size_t>(n) * nq + head) * dk + e, out);
   else if (slot >= 0) Vec4<TC>::store(k_cache + ((static_cast<size_t>(page) * nkv + (head - nq)) * page_size + off) * dk + e, out);
-}
-
-// A thread a channel, the rows of the new state in ascending order: row i takes the step's row len - (T - 1) + i of the
-// request or, where the step is shorter than that, the old state's row i + len, which lies further on and is still old.
-__global__ __launch_bounds__(kThreads) void conv_state_update_kernel(ConvIn in, float* __restrict__ state,
-                                                                     const int* __restrict__ state_slots,
-                                                                     const int* __restrict__ q_start) {
-  const int s = blockIdx.x, first = q_start[s], len = q_start[s + 1] - first, keep = in.taps - 1;
-  float* st = state + static_cast<size_t>(state_slots[s]) * keep * in.channels;
-  for (int ch = blockIdx.y * kThreads + threadIdx.x; ch < in.channels; ch += gridDim.y * kThreads)
-    for (int i = 0; i < keep; ++i) {
-      const int r = len - keep + i;
-      st[static_cast<size_t>(i) * in.channels + ch] = r >= 0 ? product_value(in, first + r, ch)
-                                                              : st[static_cast<size_t>(i + len) * in.channels + ch];
-    }
 }
 
 }  // namespace

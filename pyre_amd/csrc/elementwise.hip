@@ -8,25 +8,25 @@
 using namespace pyre;
 
 // ---------------------------------------------------------------------------
-// Embedding: out[n, :] = float(table[ids[n], :])           (pyre/model.py:196)
+// Embedding: out[n, :] = float(table[ids[n], :]) * scale   (pyre/model.py:196)
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids,
-                             float* __restrict__ out, int hidden) {
+                             float* __restrict__ out, int hidden, float scale) {
   const int n = blockIdx.x;
   const T* row = table + static_cast<size_t>(ids[n]) * hidden;
   float* o = out + static_cast<size_t>(n) * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = to_float(row[i]);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = to_float(row[i]) * scale;
 }
 
 extern "C" int pyre_embed(const void* table, int table_dt, const int* ids, float* out, int n,
-                          int hidden, hipStream_t stream) {
+                          int hidden, float scale, hipStream_t stream) {
   PYRE_REQUIRE(known_dtype(table_dt), "embed: unknown table dtype %d", table_dt);
   PYRE_REQUIRE(n >= 0 && hidden > 0, "embed: bad sizes n=%d hidden=%d", n, hidden);
   if (n == 0) return 0;
   PYRE_DISPATCH(table_dt, T,
                 hipLaunchKernelGGL(embed_kernel<T>, dim3(n), dim3(256), 0, stream,
-                                   static_cast<const T*>(table), ids, out, hidden));
+                                   static_cast<const T*>(table), ids, out, hidden, scale));
   return check_launch("embed");
 }
 

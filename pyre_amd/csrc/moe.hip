@@ -4,6 +4,9 @@
 //                s (the lower index among equals), each weighted s / (sum of the chosen s + 1e-20); written as a
 //                dense row gates[n, experts] (0 for an expert that is not chosen), float32. The experts are compared
 //                by z, which orders them as s does and still tells two apart where both their s round to one.
+//                In its softmax form the chosen experts' weights are the softmax over their logits alone. Columns of
+//                the product behind the experts' (`extra`) are gates of their own: their sigmoid is written behind
+//                the experts' weights (a shared expert's gate per token).
 //   expert_act   the experts' way up is one product over [W_0; W_1; ...; W_shared]; its result becomes
 //                act[n, e ff + j] = gates[n, e] f(up[n, e ff + j]) for the routed experts and f(up) for the columns
 //                of the shared expert behind them, f(u) = max(u, 0)^2. One product over
@@ -31,8 +34,9 @@ constexpr int kMaxPerLane = 8;  // experts a lane keeps: up to 512 experts
 
 __global__ __launch_bounds__(kWave) void route_topk_kernel(const void* __restrict__ z, int z_dt, int n_partials,
                                                            size_t partial_stride, const void* __restrict__ bias,
-                                                           int bias_dt, float* __restrict__ gates, int experts, int top) {
-  const int n = blockIdx.x, lane = threadIdx.x;
+                                                           int bias_dt, float* __restrict__ gates, int experts, int top,
+                                                           int softmax, int extra) {
+  const int n = blockIdx.x, lane = threadIdx.x, width = experts + extra;
   float s[kMaxPerLane], w[kMaxPerLane];  // s: the logits still to choose from
 #pragma unroll
   for (int u = 0; u < kMaxPerLane; ++u) {
@@ -40,12 +44,19 @@ __global__ __launch_bounds__(kWave) void route_topk_kernel(const void* __restric
     s[u] = -INFINITY, w[u] = 0.f;
     if (e < experts) {
       float v = 0.f;
-      for (int p = 0; p < n_partials; ++p) v += load_as_float(z, z_dt, p * partial_stride + static_cast<size_t>(n) * experts + e);
+      for (int p = 0; p < n_partials; ++p) v += load_as_float(z, z_dt, p * partial_stride + static_cast<size_t>(n) * width + e);
       if (bias) v += load_as_float(bias, bias_dt, e);
       s[u] = fmaxf(v, -3.0e38f);  // finite, so that it beats the mark of an expert that is taken or not there
     }
   }
-  float total = 0.f;
+  // the columns behind the experts: gates of their own, sigmoid of the logit
+  for (int e = experts + lane; e < width; e += kWave) {
+    float v = 0.f;
+    for (int p = 0; p < n_partials; ++p) v += load_as_float(z, z_dt, p * partial_stride + static_cast<size_t>(n) * width + e);
+    if (bias) v += load_as_float(bias, bias_dt, e);
+    gates[static_cast<size_t>(n) * width + e] = 1.f / (1.f + expf(-v));
+  }
+  float total = 0.f, first = 0.f;
   for (int k = 0; k < top; ++k) {
     float best = -INFINITY;
     int at = experts;
@@ -58,17 +69,18 @@ __global__ __launch_bounds__(kWave) void route_topk_kernel(const void* __restric
       const int oa = __shfl_xor(at, o, kWave);
       if (ob > best || (ob == best && oa < at)) best = ob, at = oa;
     }
-    const float score = 1.f / (1.f + expf(-best));
+    if (k == 0) first = best;  // the largest logit: the softmax over the chosen ones is taken relative to it
+    const float score = softmax ? expf(best - first) : 1.f / (1.f + expf(-best));
     total += score;
 #pragma unroll
     for (int u = 0; u < kMaxPerLane; ++u)
       if (at == lane + kWave * u) w[u] = score, s[u] = -INFINITY;
   }
-  const float inv = 1.f / (total + 1e-20f);
+  const float inv = 1.f / (softmax ? total : total + 1e-20f);
 #pragma unroll
   for (int u = 0; u < kMaxPerLane; ++u) {
     const int e = lane + kWave * u;
-    if (e < experts) gates[static_cast<size_t>(n) * experts + e] = w[u] * inv;
+    if (e < experts) gates[static_cast<size_t>(n) * width + e] = w[u] * inv;
   }
 }
 
@@ -197,16 +209,24 @@ __global__ __launch_bounds__(kWave) void route_grouped_kernel(const void* __rest
   }
 }
 
-// act[n, e ff + j] = gates[n, e] * silu(g) * u, g and u the columns e ff + j and experts ff + e ff + j of the product.
+// act[n, e ff + j] = gates[n, e] * silu(g) * u, g and u the columns e ff + j and width + e ff + j of the product
+// (width = experts ff + shared_ff: the columns behind the routed experts' are a shared expert's, of a size of its own,
+// whose weight is gates[n, shared_gate], or one if shared_gate < 0).
+__device__ inline float expert_weight(const float* gates, int e, int experts, int shared_gate) {
+  if (e < experts) return gates[e];
+  return shared_gate >= 0 ? gates[shared_gate] : 1.f;
+}
+
 __global__ __launch_bounds__(256) void expert_glu_act_kernel(const void* __restrict__ gu, int gu_dt, int n_partials,
                                                              size_t partial_stride, const float* __restrict__ gates,
                                                              size_t gates_stride, void* __restrict__ out, int out_dt,
-                                                             size_t total, int ff, int width) {
+                                                             size_t total, int ff, int width, int experts,
+                                                             int shared_gate) {
   const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= total) return;
   const size_t n = i / width;
   const int c = static_cast<int>(i % width);
-  const float w = gates[n * gates_stride + c / ff];
+  const float w = expert_weight(gates + n * gates_stride, c / ff, experts, shared_gate);
   float y = 0.f;
   if (w != 0.f) {
     float g = 0.f, u = 0.f;
@@ -223,13 +243,14 @@ __global__ __launch_bounds__(256) void expert_glu_act_kernel(const void* __restr
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void expert_glu_act_vec_kernel(const TI* __restrict__ gu, int n_partials, size_t partial_stride,
                                                                  const float* __restrict__ gates, size_t gates_stride,
-                                                                 TO* __restrict__ out, size_t total4, int ff, int width) {
+                                                                 TO* __restrict__ out, size_t total4, int ff, int width,
+                                                                 int experts, int shared_gate) {
   const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= total4) return;
   const int per_row = width / 4;
   const size_t n = i / per_row;
   const int c = 4 * static_cast<int>(i % per_row);
-  const float w = gates[n * gates_stride + c / ff];
+  const float w = expert_weight(gates + n * gates_stride, c / ff, experts, shared_gate);
   float4 y = {0.f, 0.f, 0.f, 0.f};
   if (w != 0.f) {
     const float4 g = sum_partials4(gu + n * 2 * width + c, partial_stride, n_partials);
@@ -256,13 +277,13 @@ __global__ __launch_bounds__(256) void add_weighted_rows_kernel(float* __restric
 }  // namespace
 
 extern "C" int pyre_route_topk(const void* z, int z_dt, int n_partials, long partial_stride, const void* bias, int bias_dt,
-                               float* gates, int n, int experts, int top, hipStream_t stream) {
+                               float* gates, int n, int experts, int top, int softmax, int extra, hipStream_t stream) {
   PYRE_REQUIRE(known_dtype(z_dt) && n_partials >= 1 && (!bias || known_dtype(bias_dt)), "route_topk: bad dtypes");
-  PYRE_REQUIRE(experts > 0 && experts <= kWave * kMaxPerLane && top > 0 && top <= experts,
+  PYRE_REQUIRE(experts > 0 && experts <= kWave * kMaxPerLane && top > 0 && top <= experts && extra >= 0,
                "route_topk: %d of %d experts is not a choice this kernel makes", top, experts);
   if (n <= 0) return 0;
   hipLaunchKernelGGL(route_topk_kernel, dim3(n), dim3(kWave), 0, stream, z, z_dt, n_partials,
-                     static_cast<size_t>(partial_stride), bias, bias_dt, gates, experts, top);
+                     static_cast<size_t>(partial_stride), bias, bias_dt, gates, experts, top, softmax, extra);
   return check_launch("route_topk");
 }
 
@@ -301,23 +322,25 @@ extern "C" int pyre_route_grouped(const void* z, int z_dt, int n_partials, long 
 }
 
 extern "C" int pyre_expert_glu_act(const void* gu, int gu_dt, int n_partials, long partial_stride, const float* gates,
-                                   long gates_stride, void* out, int out_dt, int n, int experts, int ff, hipStream_t stream) {
+                                   long gates_stride, void* out, int out_dt, int n, int experts, int ff, int shared_ff,
+                                   int shared_gate, hipStream_t stream) {
   PYRE_REQUIRE(known_dtype(gu_dt) && known_dtype(out_dt) && n_partials >= 1, "expert_glu_act: bad dtypes");
-  PYRE_REQUIRE(experts > 0 && ff > 0 && gates && gates_stride >= experts, "expert_glu_act: bad sizes");
+  PYRE_REQUIRE(experts > 0 && ff > 0 && shared_ff >= 0 && gates && gates_stride >= experts && shared_gate < gates_stride,
+               "expert_glu_act: bad sizes");
   if (n <= 0) return 0;
-  const int width = experts * ff;
+  const int width = experts * ff + shared_ff;
   const size_t total = static_cast<size_t>(n) * width;
-  if (ff % 4 == 0 && partial_stride % 4 == 0 && reinterpret_cast<uintptr_t>(gu) % 16 == 0 &&
+  if (ff % 4 == 0 && shared_ff % 4 == 0 && partial_stride % 4 == 0 && reinterpret_cast<uintptr_t>(gu) % 16 == 0 &&
       reinterpret_cast<uintptr_t>(out) % 16 == 0) {
     PYRE_DISPATCH(gu_dt, TI, PYRE_DISPATCH(out_dt, TO,
         hipLaunchKernelGGL((expert_glu_act_vec_kernel<TI, TO>), dim3((total / 4 + 255) / 256), dim3(256), 0, stream,
                            static_cast<const TI*>(gu), n_partials, static_cast<size_t>(partial_stride), gates,
-                           static_cast<size_t>(gates_stride), static_cast<TO*>(out), total / 4, ff, width)));
+                           static_cast<size_t>(gates_stride), static_cast<TO*>(out), total / 4, ff, width, experts, shared_gate)));
     return check_launch("expert_glu_act");
   }
   hipLaunchKernelGGL(expert_glu_act_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, gu, gu_dt, n_partials,
                      static_cast<size_t>(partial_stride), gates, static_cast<size_t>(gates_stride), out, out_dt, total, ff,
-                     width);
+                     width, experts, shared_gate);
   return check_launch("expert_glu_act");
 }
 

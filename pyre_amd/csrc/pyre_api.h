@@ -21,7 +21,8 @@ const char* pyre_sources_digest();
 // a measurement of achievable read bandwidth.
 int pyre_read_probe(const void* p, size_t bytes, int blocks, unsigned* sink, hipStream_t stream);
 
-int pyre_embed(const void* table, int table_dt, const int* ids, float* out, int n, int hidden,
+// out[n] = table[ids[n]] * scale, float32.
+int pyre_embed(const void* table, int table_dt, const int* ids, float* out, int n, int hidden, float scale,
                hipStream_t stream);
 
 int pyre_add_rmsnorm(float* resid, const void* delta, int delta_dt, int n_partials,
@@ -307,9 +308,11 @@ int pyre_head_matmul(const void* x, int x_ld, const void* w, void* out, int out_
                      int dout, hipStream_t stream);
 
 // ---- a mixture of experts with a sigmoid router (moe.hip) ----
-// gates[n, experts] float32: s / (sum of the chosen s + 1e-20) for the `top` experts of largest s = sigmoid(z), else 0.
+// gates[n, experts + extra] float32: for the `top` experts of largest logit z, s / (sum of the chosen s + 1e-20) with
+// s = sigmoid(z), or (softmax) the softmax over the chosen logits alone; 0 for the others; sigmoid(z) for the `extra`
+// columns behind the experts, which are gates of their own.
 int pyre_route_topk(const void* z, int z_dt, int n_partials, long partial_stride, const void* bias, int bias_dt,
-                    float* gates, int n, int experts, int top, hipStream_t stream);
+                    float* gates, int n, int experts, int top, int softmax, int extra, hipStream_t stream);
 // out[n, e ff + j] = gates[n, e] max(up, 0)^2 for e < experts, max(up, 0)^2 for the shared_ff columns behind them.
 int pyre_expert_act(const void* up, int up_dt, int n_partials, long partial_stride, const float* gates, void* out,
                     int out_dt, int n, int experts, int ff, int shared_ff, hipStream_t stream);
@@ -344,8 +347,36 @@ int pyre_retention_prepare(const void* proj, int proj_dt, int n_partials, long p
 int pyre_route_grouped(const void* z, int z_dt, int n_partials, long partial_stride, const void* bias, int bias_dt,
                        const float* correction, float* gates, int n, int experts, int top, int groups, int keep_groups,
                        hipStream_t stream);
+// The experts' gated units, weighted; behind them shared_ff columns of a shared expert, weighted by gates[n, shared_gate]
+// (shared_gate < 0: by one).
 int pyre_expert_glu_act(const void* gu, int gu_dt, int n_partials, long partial_stride, const float* gates,
-                        long gates_stride, void* out, int out_dt, int n, int experts, int ff, hipStream_t stream);
+                        long gates_stride, void* out, int out_dt, int n, int experts, int ff, int shared_ff,
+                        int shared_gate, hipStream_t stream);
 int pyre_add_weighted_rows(float* p, const void* h, int h_dt, long h_stride, const float* gates, long gates_stride,
                            int first, int count, int n, int width, hipStream_t stream);
+
+// The input product of an attention whose queries and keys are normed over their whole projection (wide_norm_qkv.hip).
+int pyre_wide_norm_qkv_write(const void* proj, int proj_dt, int n_partials, long partial_stride, int ld, int col0,
+                             const float* bias, const float* q_gain, const float* k_gain, float eps, const float* cos,
+                             const float* sin, int rot, const int* positions, void* q_out, int q_dt, void* k_cache,
+                             void* v_cache, int cache_dt, const int* slots, int n, int nq, int nkv, int dk, int dv,
+                             int page_size, int write_kv, hipStream_t stream);
+
+// ---- the gated delta rule (delta_rule.hip) ----
+// Columns of the float32 rows [q | k | decay | v | gate | beta] that its kernels share.
+long pyre_gdr_row_width(int H, int G, int dk, int dv);
+int pyre_gdr_prepare(const void* proj, int proj_dt, int n_partials, long partial_stride, int ld, int col0,
+                     const float* bias, const float* taps_w, int taps, float* conv_state, const int* state_slots,
+                     const int* seq_of_token, const int* q_start, int n_seqs, const void* a2, int a2_dt,
+                     const float* dt_bias, const float* rate, const void* g2, int g2_dt, float unit_eps, float* x, int n,
+                     int H, int G, int dk, int dv, int rank_a, int rank_g, hipStream_t stream);
+int pyre_gdr_scan(const float* x, float* state, float* o, const int* q_start, const int* state_slots, int n_seqs, int H,
+                  int G, int dk, int dv, hipStream_t stream);
+int pyre_gdr_finish(const float* o, const float* x, const void* gain, int gain_dt, float eps, float out_scale, void* out,
+                    int out_dt, long out_ld, int n, int H, int G, int dk, int dv, hipStream_t stream);
+
+// out[n, j] = gelu_tanh(z[n, j]) * table[ids[n], first + j], z the partial sums of a product [n, dim] (token_side.hip).
+int pyre_token_side_gate(const void* z, int z_dt, int n_partials, long partial_stride, const void* bias, int bias_dt,
+                         const void* table, int table_dt, int table_width, int first, const int* ids, void* out,
+                         int out_dt, int n, int dim, hipStream_t stream);
 }  // extern "C"

@@ -11,7 +11,7 @@ from ctypes import c_float, c_int, c_long, c_void_p
 
 from pyre_amd.hip import build as _build
 
-ABI_VERSION = 27
+ABI_VERSION = 28
 
 
 class KernelError(RuntimeError):
@@ -22,7 +22,7 @@ P, I, L, F = c_void_p, c_int, c_long, c_float
 
 _SIGNATURES = {
     "pyre_read_probe": [P, ctypes.c_size_t, I, P, P],
-    "pyre_embed": [P, I, P, P, I, I, P],
+    "pyre_embed": [P, I, P, P, I, I, F, P],
     "pyre_add_rmsnorm": [P, P, I, I, L, P, I, P, I, P, I, P, I, I, F, P],
     "pyre_rope_kv_write": [P, I, I, L, P, I, P, I, P, P, I, P, P, I, P, P, I, I, I, I, I, I, P],
     "pyre_silu_mul": [P, I, I, L, P, I, I, I, P],
@@ -72,7 +72,7 @@ _SIGNATURES = {
     "pyre_rope_tied_write": [P, I, I, L, I, I, P, I, P, I, P, P, I, P, P, I, P, P, I, I, I, I, I, I, P],
     "pyre_latent_write": [P, I, I, L, I, I, P, I, P, I, P, I, F, P, I, I, I, I, I, P],
     "pyre_head_matmul": [P, I, P, P, I, I, I, I, I, I, P],
-    "pyre_route_topk": [P, I, I, L, P, I, P, I, I, I, P],
+    "pyre_route_topk": [P, I, I, L, P, I, P, I, I, I, I, I, P],
     "pyre_expert_act": [P, I, I, L, P, P, I, I, I, I, I, P],
     "pyre_add_rms_terms": [P, P, I, I, L, P, I, F, P, I, I, L, P, I, F, F, P, I, F, P, I, F, P, I, P, I, I, P],
     "pyre_bigram_embed": [P, P, I, P, P, P, P, P, P, P, I, I, I, I, I, P],
@@ -80,8 +80,13 @@ _SIGNATURES = {
                             I, I, I, P],
     "pyre_retention_prepare": [P, I, I, L, I, I, P, P, P, I, I, P, F, P, I, I, I, I, P],
     "pyre_route_grouped": [P, I, I, L, P, I, P, P, I, I, I, I, I, P],
-    "pyre_expert_glu_act": [P, I, I, L, P, L, P, I, I, I, I, P],
+    "pyre_expert_glu_act": [P, I, I, L, P, L, P, I, I, I, I, I, I, P],
     "pyre_add_weighted_rows": [P, P, I, L, P, L, I, I, I, I, P],
+    "pyre_wide_norm_qkv_write": [P, I, I, L, I, I, P, P, P, F, P, P, I, P, P, I, P, P, I, P, I, I, I, I, I, I, I, P],
+    "pyre_gdr_prepare": [P, I, I, L, I, I, P, P, I, P, P, P, P, I, P, I, P, P, P, I, F, P, I, I, I, I, I, I, I, P],
+    "pyre_gdr_scan": [P, P, P, P, P, I, I, I, I, I, P],
+    "pyre_gdr_finish": [P, P, P, I, F, F, P, I, L, I, I, I, I, I, P],
+    "pyre_token_side_gate": [P, I, I, L, P, I, P, I, I, I, P, P, I, I, I, P],
 }
 
 _lib = None

@@ -122,15 +122,15 @@ class Partials:
                 _ptr(self.bias), dtype_code(self.bias) if self.bias is not None else 0)
 
 
-def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
-    """out[n] = float32(table[ids[n]]); ids must already be checked against the vocabulary."""
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+    """out[n] = float32(table[ids[n]]) * scale; ids must already be checked against the vocabulary."""
     _dev(table, ids, out)
     n, hidden = out.shape
     if table.dim() != 2 or table.shape[1] != hidden or out.dtype != torch.float32:
         raise KernelError("embed: table [V, H] and float32 out [N, H] expected")
     _contig("table", table), _contig("out", out), _i32("ids", ids, n)
     call("pyre_embed", table.data_ptr(), dtype_code(table), ids.data_ptr(), out.data_ptr(), n, hidden,
-         _stream())
+         float(scale), _stream())
 
 
 def add_rmsnorm(resid: torch.Tensor, delta: Partials | None, gain: torch.Tensor, eps: float,
@@ -1116,17 +1116,20 @@ def head_matmul(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n: int) -> 
 ROUTE_MAX_EXPERTS = 512  #: the most experts that the routing kernel chooses among (moe.hip)
 
 
-def route_topk(z: Partials, gates: torch.Tensor, n: int, top: int) -> None:
-    """gates[n, e] (float32 [N, experts]) = s_e / (sum of the chosen s + 1e-20) for the ``top`` experts of largest
-    s = sigmoid(z) (the lower index among equals), 0 for the others; ``z`` the router product's partial sums."""
+def route_topk(z: Partials, gates: torch.Tensor, n: int, top: int, softmax: bool = False, extra: int = 0) -> None:
+    """gates[n, e] (float32 [N, experts + extra]) = s_e / (sum of the chosen s + 1e-20) for the ``top`` experts of largest
+    s = sigmoid(z) (the lower index among equals), 0 for the others; ``z`` the router product's partial sums.
+    ``softmax``: the chosen experts' weights are the softmax over their logits alone. The last ``extra`` columns of the
+    product are no experts but gates of their own, whose sigmoid is written behind the experts' weights."""
     _dev(z.data, z.bias, gates)
-    experts = z.width
-    if gates.dtype != torch.float32 or not gates.is_contiguous() or gates.dim() != 2 or gates.shape[1] != experts or \
+    experts = z.width - int(extra)
+    if gates.dtype != torch.float32 or not gates.is_contiguous() or gates.dim() != 2 or gates.shape[1] != z.width or \
             gates.shape[0] < n or z.rows < n:
-        raise KernelError("route_topk: gates are contiguous float32 [>= n, experts]")
-    if not (0 < top <= experts <= ROUTE_MAX_EXPERTS):
+        raise KernelError("route_topk: gates are contiguous float32 [>= n, experts + extra]")
+    if extra < 0 or not (0 < top <= experts <= ROUTE_MAX_EXPERTS):
         raise KernelError(f"route_topk: {top} of {experts} experts is not a choice this kernel makes")
-    call("pyre_route_topk", *z._args(experts), gates.data_ptr(), n, experts, int(top), _stream())
+    call("pyre_route_topk", *z._args(z.width), gates.data_ptr(), n, experts, int(top), int(bool(softmax)), int(extra),
+         _stream())
 
 
 def expert_act(up: Partials, gates: torch.Tensor, out: torch.Tensor, n: int, experts: int, ff: int, shared_ff: int) -> None:
@@ -1344,21 +1347,25 @@ def route_grouped(z: Partials, correction: torch.Tensor | None, gates: torch.Ten
          int(keep_groups), _stream())
 
 
-def expert_glu_act(gu: Partials, gates: torch.Tensor, out: torch.Tensor, n: int, experts: int, ff: int) -> None:
-    """out[n, e*ff + j] = gates[n, e] * silu(g) * u with g = gu[n, e*ff + j] and u = gu[n, experts*ff + e*ff + j]: the
+def expert_glu_act(gu: Partials, gates: torch.Tensor, out: torch.Tensor, n: int, experts: int, ff: int,
+                   shared_ff: int = 0, shared_gate: int = -1) -> None:
+    """out[n, e*ff + j] = gates[n, e] * silu(g) * u with g = gu[n, e*ff + j] and u = gu[n, width + e*ff + j]: the
     experts' gated units, weighted (``gates [N, >= experts]`` with contiguous rows; columns of an expert that the token
-    does not take are not read and written as zero)."""
+    does not take are not read and written as zero). ``shared_ff`` columns behind the routed experts' (width = experts*ff
+    + shared_ff) are a shared expert's, weighted by ``gates[n, shared_gate]`` (``shared_gate`` < 0: by one)."""
     _dev(gu.data, gates, out)
-    width = experts * ff
+    width = experts * ff + shared_ff
+    if shared_ff < 0 or shared_gate >= gates.shape[1]:
+        raise KernelError("expert_glu_act: the shared expert's gate lies outside the rows of weights")
     if gu.bias is not None:
         raise KernelError("expert_glu_act: a pending bias is not supported")
     if gu.width != 2 * width or gu.rows < n or out.shape[-1] != width or out.shape[0] < n:
-        raise KernelError("expert_glu_act: the product's width does not fit 2 * experts * ff")
+        raise KernelError("expert_glu_act: the product's width does not fit 2 * (experts * ff + shared_ff)")
     if gates.dtype != torch.float32 or gates.dim() != 2 or gates.stride(1) != 1 or gates.shape[1] < experts or gates.shape[0] < n:
         raise KernelError("expert_glu_act: gates are float32 [>= n, >= experts] with contiguous rows")
     _contig("out", out)
     call("pyre_expert_glu_act", gu.data.data_ptr(), dtype_code(gu.data), gu.count, gu.stride, gates.data_ptr(),
-         gates.stride(0), out.data_ptr(), dtype_code(out), n, experts, ff, _stream())
+         gates.stride(0), out.data_ptr(), dtype_code(out), n, experts, ff, int(shared_ff), int(shared_gate), _stream())
 
 
 def add_weighted_rows(p: Partials, h: torch.Tensor, gates: torch.Tensor, first: int, count: int, n: int) -> None:
@@ -1386,3 +1393,150 @@ def relu2(up: Partials, out: torch.Tensor, n: int) -> None:
     _contig("out", out)
     call("pyre_expert_act", up.data.data_ptr(), dtype_code(up.data), up.count, up.stride, None,
          out.data_ptr(), dtype_code(out), n, 0, 4, up.width, _stream())
+
+
+def _proj_bias_args(proj: Partials, col0: int, width: int):
+    """As :func:`_proj_args` for the kernels that add the product's pending bias themselves: float32 over all its columns."""
+    if col0 < 0 or col0 + width > proj.width:
+        raise KernelError(f"columns {col0}..{col0 + width} lie outside the product's {proj.width}")
+    bias = proj.bias
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != proj.width or not bias.is_contiguous()):
+        raise KernelError(f"a fused input product's bias is contiguous float32 [{proj.width}]")
+    _dev(proj.data, bias)
+    return (proj.data.data_ptr(), dtype_code(proj.data), proj.count, proj.stride, proj.width, col0, _ptr(bias))
+
+
+def _rot_tables(what: str, cos, sin, rot: int, dk: int):
+    if not rot:
+        return None, None
+    if rot % 2 or rot > dk or cos is None or sin is None or cos.dtype != torch.float32 or sin.dtype != torch.float32 \
+            or cos.dim() != 2 or cos.shape[1] != rot // 2 or tuple(cos.shape) != tuple(sin.shape):
+        raise KernelError(f"{what}: cos and sin are float32 [positions, rot / 2], rot even and within the head")
+    _contig("cos", cos), _contig("sin", sin)
+    return cos.data_ptr(), sin.data_ptr()
+
+
+def wide_norm_qkv_write(proj: Partials, col0: int, q_gain: torch.Tensor | None, k_gain: torch.Tensor | None, eps: float,
+                        cos: torch.Tensor | None, sin: torch.Tensor | None, rot: int, positions: torch.Tensor,
+                        q_out: torch.Tensor, k_cache: torch.Tensor | None, v_cache: torch.Tensor | None,
+                        slots: torch.Tensor | None, n: int, nq: int, nkv: int, dk: int, dv: int, page_size: int) -> None:
+    """Finish a step's input product from column ``col0`` on (``nq`` query heads of ``dk``, then ``nkv`` key heads of ``dk``
+    and ``nkv`` value heads of ``dv``; ``nkv`` = 0: queries alone), its pending bias included. Queries are divided by their
+    root mean square over all ``nq * dk`` columns at once, times ``q_gain`` over those columns (None: not normed), keys
+    likewise over their ``nkv * dk`` with ``k_gain``; then the first ``rot`` elements of every head are turned by position,
+    element e with e + rot/2. Queries go to ``q_out [N, nq*dk]``, keys and values to their pages at ``slots``
+    (``k_cache`` None: nothing is stored)."""
+    _dev(q_gain, k_gain, cos, sin, positions, q_out, k_cache, v_cache, slots)
+    args = _proj_bias_args(proj, col0, (nq + nkv) * dk + nkv * dv)
+    if proj.rows < n or q_out.numel() < n * nq * dk:
+        raise KernelError("wide_norm_qkv_write: buffers are smaller than the batch")
+    _contig("q_out", q_out), _i32("positions", positions, n)
+    for name, g, width in (("q_gain", q_gain, nq * dk), ("k_gain", k_gain, nkv * dk)):
+        if g is not None and (g.dtype != torch.float32 or g.numel() != width or not g.is_contiguous()):
+            raise KernelError(f"wide_norm_qkv_write: {name} is contiguous float32 [{width}]")
+    c, s = _rot_tables("wide_norm_qkv_write", cos, sin, rot, dk)
+    write = k_cache is not None
+    cache_dt = dtype_code(q_out)
+    if write:
+        if v_cache is None or slots is None or nkv <= 0:
+            raise KernelError("wide_norm_qkv_write: k cache without v cache, slots or key heads")
+        _i32("slots", slots, n), _contig("k_cache", k_cache), _contig("v_cache", v_cache)
+        if tuple(k_cache.shape[1:]) != (nkv, page_size, dk) or tuple(v_cache.shape[1:]) != (nkv, page_size, dv) \
+                or k_cache.dtype != v_cache.dtype:
+            raise KernelError(f"wide_norm_qkv_write: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} do not fit "
+                              f"nkv={nkv} page={page_size} dk={dk} dv={dv}")
+        cache_dt = dtype_code(k_cache)
+    call("pyre_wide_norm_qkv_write", *args, _ptr(q_gain), _ptr(k_gain), float(eps), c, s, int(rot), positions.data_ptr(),
+         q_out.data_ptr(), dtype_code(q_out), _ptr(k_cache), _ptr(v_cache), cache_dt, _ptr(slots), n, nq, nkv, dk, dv,
+         page_size, 1 if write else 0, _stream())
+
+
+GDR_MAX_HEAD = 256   #: the largest key or value head of the gated delta rule's kernels (delta_rule.hip)
+GDR_MAX_RANK = 512   #: the widest low-rank input of its decay and of its gate
+
+
+def gdr_row_width(heads: int, kv_heads: int, dk: int, dv: int) -> int:
+    """Columns of the float32 rows [q | k | decay | v | gate | beta] that the gated delta rule's kernels share."""
+    return 2 * kv_heads * dk + heads * dk + 2 * heads * dv + heads
+
+
+def gdr_prepare(proj: Partials, col0: int, taps_w: torch.Tensor | None, conv_state: torch.Tensor | None,
+                state_slots: torch.Tensor, seq_of_token: torch.Tensor, q_start: torch.Tensor, n_seqs: int,
+                a2: torch.Tensor, dt_bias: torch.Tensor, rate: torch.Tensor, g2: torch.Tensor, unit_eps: float,
+                x: torch.Tensor, n: int, heads: int, kv_heads: int, dk: int, dv: int) -> None:
+    """Finish the input product from column ``col0`` on (q, k: kv_heads*dk each; v: heads*dv; beta: heads; then the low-rank
+    inputs of the decay and of the gate) into the float32 rows ``x``: q, k, v through the short causal convolution
+    (``taps_w`` float32 [taps, channels], inputs before the step from ``conv_state [slots, taps - 1, channels]``, which is
+    brought up to date afterwards) and SiLU; q and k unit vectors per head (``unit_eps`` beside the sum of squares), q times
+    dk^-1/2; beta = sigmoid; decay = exp(rate[h] * softplus(a2 @ low + dt_bias)); gate = sigmoid(g2 @ low')."""
+    _dev(taps_w, conv_state, state_slots, seq_of_token, q_start, a2, dt_bias, rate, g2, x)
+    rank_a, rank_g = a2.shape[1], g2.shape[1]
+    channels = 2 * kv_heads * dk + heads * dv
+    args = _proj_bias_args(proj, col0, channels + heads + rank_a + rank_g)
+    if tuple(a2.shape) != (heads * dk, rank_a) or tuple(g2.shape) != (heads * dv, rank_g):
+        raise KernelError("gdr_prepare: the second matrices are [heads*dk, rank] and [heads*dv, rank']")
+    _contig("a2", a2), _contig("g2", g2)
+    for name, t, size in (("dt_bias", dt_bias, heads * dk), ("rate", rate, heads)):
+        if t.dtype != torch.float32 or t.numel() != size or not t.is_contiguous():
+            raise KernelError(f"gdr_prepare: {name} is contiguous float32 [{size}]")
+    if x.dtype != torch.float32 or not x.is_contiguous() or x.shape[-1] != gdr_row_width(heads, kv_heads, dk, dv) or \
+            x.shape[0] < n or proj.rows < n:
+        raise KernelError("gdr_prepare: x is contiguous float32 [>= n, gdr_row_width(...)]")
+    _i32("seq_of_token", seq_of_token, n), _i32("q_start", q_start, n_seqs + 1), _i32("state_slots", state_slots, n_seqs)
+    taps = 0
+    if taps_w is not None:
+        taps = taps_w.shape[0]
+        if taps_w.dtype != torch.float32 or not taps_w.is_contiguous() or tuple(taps_w.shape) != (taps, channels) or \
+                not (1 <= taps <= CONV_MAX_TAPS):
+            raise KernelError(f"gdr_prepare: the taps are contiguous float32 [1..{CONV_MAX_TAPS}, {channels}]")
+        if taps > 1 and (conv_state is None or conv_state.dtype != torch.float32 or not conv_state.is_contiguous() or
+                         tuple(conv_state.shape[1:]) != (taps - 1, channels)):
+            raise KernelError(f"gdr_prepare: the state is contiguous float32 [slots, {taps - 1}, {channels}]")
+    call("pyre_gdr_prepare", *args, _ptr(taps_w), taps, _ptr(conv_state) if taps > 1 else None, state_slots.data_ptr(),
+         seq_of_token.data_ptr(), q_start.data_ptr(), n_seqs, a2.data_ptr(), dtype_code(a2), dt_bias.data_ptr(),
+         rate.data_ptr(), g2.data_ptr(), dtype_code(g2), float(unit_eps), x.data_ptr(), n, heads, kv_heads, dk, dv,
+         rank_a, rank_g, _stream())
+
+
+def gdr_scan(x: torch.Tensor, state: torch.Tensor, o: torch.Tensor, q_start: torch.Tensor, state_slots: torch.Tensor,
+             n_seqs: int, heads: int, kv_heads: int, dk: int, dv: int) -> None:
+    """The gated delta rule over each request's tokens of the step, from and into ``state [slots, heads, dk, dv]``:
+    S <- diag(decay) S; u = beta (v - S^T k); S <- S + k u^T; ``o`` (float32 [N, heads*dv]) receives S^T q."""
+    _dev(x, state, o, q_start, state_slots)
+    for name, t in (("x", x), ("state", state), ("o", o)):
+        if t.dtype != torch.float32 or not t.is_contiguous():
+            raise KernelError(f"gdr_scan: {name} is contiguous float32")
+    if tuple(state.shape[1:]) != (heads, dk, dv) or x.shape[-1] != gdr_row_width(heads, kv_heads, dk, dv) or \
+            o.shape[-1] != heads * dv:
+        raise KernelError("gdr_scan: shapes do not fit the head geometry")
+    _i32("q_start", q_start, n_seqs + 1), _i32("state_slots", state_slots, n_seqs)
+    call("pyre_gdr_scan", x.data_ptr(), state.data_ptr(), o.data_ptr(), q_start.data_ptr(), state_slots.data_ptr(), n_seqs,
+         heads, kv_heads, dk, dv, _stream())
+
+
+def gdr_finish(o: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, eps: float, out_scale: float, out: torch.Tensor,
+               n: int, heads: int, kv_heads: int, dk: int, dv: int) -> None:
+    """out[n, h*dv + e] = o / rms(o over dv) * gain[e] * gate * out_scale, the gate from the rows ``x``; ``out`` has
+    contiguous rows."""
+    _dev(o, x, gain, out)
+    if o.dtype != torch.float32 or x.dtype != torch.float32 or not o.is_contiguous() or not x.is_contiguous():
+        raise KernelError("gdr_finish: o and x are contiguous float32")
+    if gain.numel() != dv or out.dim() != 2 or out.stride(1) != 1 or out.shape[1] < heads * dv or out.shape[0] < n or \
+            x.shape[-1] != gdr_row_width(heads, kv_heads, dk, dv) or o.shape[-1] != heads * dv:
+        raise KernelError("gdr_finish: gain [dv] and out [>= n, >= heads*dv] expected")
+    _contig("gain", gain)
+    call("pyre_gdr_finish", o.data_ptr(), x.data_ptr(), gain.data_ptr(), dtype_code(gain), float(eps), float(out_scale),
+         out.data_ptr(), dtype_code(out), out.stride(0), n, heads, kv_heads, dk, dv, _stream())
+
+
+def token_side_gate(z: Partials, table: torch.Tensor, first: int, ids: torch.Tensor, out: torch.Tensor, n: int) -> None:
+    """out[n, j] = gelu_tanh(z[n, j]) * table[ids[n], first + j] for the ``z.width`` columns of the narrow product ``z``."""
+    _dev(z.data, z.bias, table, ids, out)
+    dim = z.width
+    if table.dim() != 2 or not table.is_contiguous() or first < 0 or first + dim > table.shape[1]:
+        raise KernelError(f"token_side_gate: columns {first}..{first + dim} lie outside the table's {tuple(table.shape)}")
+    if out.shape[-1] != dim or out.shape[0] < n or z.rows < n:
+        raise KernelError("token_side_gate: the output does not fit the product")
+    _contig("out", out), _i32("ids", ids, n)
+    call("pyre_token_side_gate", *z._args(dim), table.data_ptr(), dtype_code(table), table.shape[1], int(first),
+         ids.data_ptr(), out.data_ptr(), dtype_code(out), n, dim, _stream())

@@ -255,7 +255,7 @@ class Block(Part):
 # --------------------------------------------------------------------------- registry of parts
 
 _PARTS: dict[tuple[str, str], type] = {}
-ROLES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head")
+ROLES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head", "token_input")
 
 
 def register_part(role: str, kind: str, cls: type) -> None:
@@ -289,6 +289,7 @@ class RMSNormSpec:
     eps: float
     prefix: str                      #: tensor name is ``prefix + ".weight"``
     name: str | None = None          #: or this, as it stands
+    one_plus: bool = False           #: the tensor is stored around zero: the gain is one plus it
     kind: ClassVar[str] = "rmsnorm"
 
     @property
@@ -310,6 +311,10 @@ class RotarySpec:
     #: instead of float32 arithmetic all the way
     exact: bool = False
     pairing: str = "halves"
+    #: (factor, original, fast, slow): the frequencies of pairs that turn fewer than ``slow`` times over ``original``
+    #: positions are divided by ``factor``, those that turn more than ``fast`` times stay, those between are blended
+    #: linearly by their index; cosines and sines are multiplied by 0.1 ln(factor) + 1. None: plain frequencies.
+    scaling: tuple | None = None
     kind: ClassVar[str] = "rotary"
 
 
@@ -540,6 +545,96 @@ class GroupedSoftmaxMoESpec:
 
 
 @dataclass(frozen=True)
+class WindowAttentionSpec:
+    """Grouped softmax attention over a window of ``window`` tokens (0: all earlier ones) with biased projections
+    (``qkv_bias``, ``out_bias``). ``wide_norm``: queries and keys are divided by their root mean square over their whole
+    projection, all heads at once, times a gain over that projection, before they are turned by position (``position``,
+    element e with e + rot/2). ``sink``: "zero" adds one term of score 0, without a value, to the softmax's denominator;
+    "none" is the ordinary softmax. ``own_kv`` False: the layer has no key and value projections and reads the pages that
+    another layer keeps (the order of layers names it). ``cache_window``: the window by which pages are given back, if it
+    has to be wider than the layer's own (a layer whose pages another reads with a wider window; 0 with a window of its
+    own: never). Tensors: ``prefix + .q / .k / .v / .o`` with ``.b`` for the biases, ``.q.norm / .k.norm``."""
+
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    key_dim: int
+    value_dim: int
+    scale: float
+    position: Any
+    prefix: str
+    window: int = 0
+    qkv_bias: bool = True
+    out_bias: bool = False
+    wide_norm: bool = False
+    norm_eps: float = 1e-6
+    sink: str = "none"
+    own_kv: bool = True
+    cache_window: int | None = None
+    kind: ClassVar[str] = "window_attention"
+
+
+@dataclass(frozen=True)
+class GatedDeltaRuleSpec:
+    """Per value head a float32 state S [key_dim, value_dim]: S <- diag(a) S; u = beta (v - S^T k); S <- S + k u^T;
+    o = S^T q. ``num_kv_heads`` query/key heads serve ``num_heads`` value heads. q, k and v go through a short causal
+    convolution (``conv_taps`` per channel, no bias) and SiLU; q and k are then unit vectors per head (``unit_eps`` beside
+    the sum of squares), q times key_dim^-1/2. beta = sigmoid(B h); a = exp(-exp(A_log_h) softplus(A2 (A1 h) + dt_bias))
+    per head and key channel; every head's o is divided by its root mean square (``norm_eps``), times a gain over
+    value_dim, times sigmoid(G2 (G1 h)). The ranks of the two low-rank products are the file's to say (None).
+    Tensors: ``prefix + .q / .k / .v / .b / .a1 / .a2 / .g1 / .g2 / .o / .q.conv / .k.conv / .v.conv / .A_log /
+    .dt_bias / .norm``."""
+
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    key_dim: int
+    value_dim: int
+    conv_taps: int
+    prefix: str
+    norm_eps: float = 1e-6
+    unit_eps: float = 1e-6
+    decay_rank: int | None = None
+    gate_rank: int | None = None
+    kind: ClassVar[str] = "gated_delta_rule"
+
+
+@dataclass(frozen=True)
+class SoftmaxTopKMoESpec:
+    """A mixture of ``experts`` gated units down(silu(gate(x)) * up(x)) of ``expert_size`` hidden units: every token goes
+    through the ``top`` experts of largest router logit (``router_bias``: the router has a bias), weighted by the softmax
+    over the chosen logits alone; a shared expert of ``shared_size`` units (0: none) runs for every token and is added,
+    times sigmoid(sg . x), one number per token (``shared_gate``). Tensors: ``prefix + .router / .router.b``,
+    ``.e<i>.gate / .up / .down``, ``.shared.gate / .up / .down / .sg``."""
+
+    hidden_size: int
+    experts: int
+    top: int
+    expert_size: int
+    prefix: str
+    shared_size: int = 0
+    shared_gate: bool = True
+    router_bias: bool = True
+    kind: ClassVar[str] = "softmax_topk_moe"
+
+
+@dataclass(frozen=True)
+class TokenSideSpec:
+    """A layer's input from the token itself: proj(gelu_tanh(gate(x)) * table[token, first : first + dim]), x the residual
+    stream. ``table`` is shared by the layers, each of which takes ``dim`` of its ``table_width`` columns. Tensors: ``table``,
+    ``prefix + .gate / .proj``."""
+
+    hidden_size: int
+    vocab_size: int
+    dim: int
+    table: str
+    table_width: int
+    first: int
+    prefix: str
+    kind: ClassVar[str] = "token_side"
+
+
+@dataclass(frozen=True)
 class PostNormBlockSpec:
     """x += post_norm(mixer(x)); x += post_norm(feed_forward(x)): the sublayers read the residual stream itself (in the
     engine's element type) and only their results are normed (RMS norms). ``feed_forward`` None: the first half alone."""
@@ -618,12 +713,16 @@ class SwiGLUSpec:
 
 @dataclass(frozen=True)
 class BlockSpec:
-    """x += mixer(norm(x)); x += feed_forward(norm(x))   (pre-norm residual block)."""
+    """x += mixer(norm(x)); x += feed_forward(norm(x))   (pre-norm residual block; ``feed_forward`` None: the first half
+    alone). ``token_input``: a third sublayer that reads the residual stream itself and the step's tokens, whose result is
+    RMS-normed (``token_input_norm``) before it joins the stream."""
 
     mixer: Any
     mixer_norm: Any
     feed_forward: Any
     feed_forward_norm: Any
+    token_input: Any = None
+    token_input_norm: Any = None
     kind: ClassVar[str] = "pre_norm"
 
 
@@ -632,6 +731,7 @@ class EmbeddingSpec:
     vocab_size: int
     hidden_size: int
     name: str = "model.embed_tokens.weight"
+    scale: float = 1.0               #: the table's rows are multiplied by this
     kind: ClassVar[str] = "embedding"
 
 

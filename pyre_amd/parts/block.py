@@ -21,17 +21,27 @@ class Hidden:
 
 
 class PreNormBlock(Block):
-    """x += mixer(norm1(x)); x += feed_forward(norm2(x))."""
+    """x += mixer(norm1(x)); x += feed_forward(norm2(x)), the second half only if the layer has a feed-forward. A layer
+    may have a third sublayer that reads the residual stream itself and the step's tokens (``token_input``): the kernel
+    that adds the pending term also writes the stream's rows in the engine's element type for it, and its result is
+    handed on with its RMS norm, which the next norm's kernel applies as it adds. A mixer made of several
+    (``cache_specs`` on the mixer) gets all of the block's cache views, a plain one its own."""
 
     def __init__(self, spec: BlockSpec):
         self.spec = spec
         self.mixer = make_part("mixer", spec.mixer)
         self.mixer_norm = make_part("norm", spec.mixer_norm)
-        self.feed_forward = make_part("feed_forward", spec.feed_forward)
-        self.feed_forward_norm = make_part("norm", spec.feed_forward_norm)
+        self.feed_forward = self.feed_forward_norm = self.token_input = self.token_input_norm = None
+        if spec.feed_forward is not None:
+            self.feed_forward = make_part("feed_forward", spec.feed_forward)
+            self.feed_forward_norm = make_part("norm", spec.feed_forward_norm)
+        if spec.token_input is not None:
+            self.token_input = make_part("token_input", spec.token_input)
+            self.token_input_norm = make_part("norm", spec.token_input_norm)
 
     def parts(self):
-        return (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward)
+        return tuple(p for p in (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward,
+                                 self.token_input, self.token_input_norm) if p is not None)
 
     def tensor_specs(self) -> list[TensorSpec]:
         return [s for p in self.parts() for s in p.tensor_specs()]
@@ -44,6 +54,8 @@ class PreNormBlock(Block):
         return [lin for p in self.parts() for lin in p.linears()]
 
     def cache_specs(self) -> list:
+        if hasattr(self.mixer, "cache_specs"):
+            return list(self.mixer.cache_specs())
         spec = self.mixer.cache_spec()
         return [] if spec is None else [spec]
 
@@ -53,9 +65,24 @@ class PreNormBlock(Block):
     def forward(self, ctx, state: Hidden, caches: list) -> None:
         h = ctx.workspace.get("block.h", (ctx.n_tokens, state.resid.shape[1]), ctx.dtype)
         self.mixer_norm.forward(ctx, state.resid, state.pending, h)
-        mixed = self.mixer.forward(ctx, h, caches[0] if caches else None)
-        self.feed_forward_norm.forward(ctx, state.resid, mixed, h)
-        state.pending = self.feed_forward.forward(ctx, h)
+        cache = caches if hasattr(self.mixer, "cache_specs") else (caches[0] if caches else None)
+        state.pending = self.mixer.forward(ctx, h, cache)
+        if self.feed_forward is not None:
+            self.feed_forward_norm.forward(ctx, state.resid, state.pending, h)
+            state.pending = self.feed_forward.forward(ctx, h)
+        if self.token_input is None:
+            return
+        from pyre_amd.hip import ops
+
+        pending = state.pending
+        if pending is not None and pending.bias is not None:  # the kernel below takes no pending bias: summed first
+            full = ctx.workspace.get("block.sum", (1, ctx.n_tokens, state.resid.shape[1]), torch.float32)
+            ops.reduce_partials(pending, full[0], ctx.n_tokens)
+            pending = Partials(full)
+        ops.add_rms_terms(state.resid, pending, None, 0.0, h)   # the pending term joins the stream; h = the stream
+        term = self.token_input.forward(ctx, h)
+        norm = self.token_input_norm
+        state.pending = Partials(term.data, term.bias, PostNorm(norm.gain, norm.spec.eps, kind="rms"))
 
 
 class SandwichBlock(Block):

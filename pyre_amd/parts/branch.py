@@ -37,6 +37,14 @@ class BranchMixer(Mixer):
     def out_tensor(self) -> TensorSpec:
         raise NotImplementedError
 
+    def in_biases(self) -> list:
+        """One entry per input matrix, in their order: the description of its bias, or None. A product with biases hands
+        them on as its pending bias (float32 over all its columns); ``attend`` must then be one that adds it."""
+        return [None] * len(self.in_tensors())
+
+    def out_bias(self) -> TensorSpec | None:
+        return None
+
     def other_tensors(self) -> list[TensorSpec]:
         return []
 
@@ -54,14 +62,16 @@ class BranchMixer(Mixer):
 
     # ---- standing alone
     def tensor_specs(self) -> list[TensorSpec]:
-        return [*self.in_tensors(), self.out_tensor(), *self.other_tensors()]
+        return [*self.in_tensors(), self.out_tensor(), *_bias_specs(self), *self.other_tensors()]
 
     def bind(self, tensors, runtime) -> None:
+        bias = _in_bias(self, tensors)
         w = _stacked([s.name for s in self.in_tensors()], tensors, 0)  # a size that only the file knows is known now
         self._in = Linear(self.hidden_size, w.shape[0], f"{self.role}.in")
         self._out = Linear(self.inner, self.hidden_size, f"{self.role}.out")
-        self._in.set(w)
-        self._out.set(take(tensors, self.out_tensor().name))
+        self._in.set(w, None if bias is None else torch.cat(bias))
+        ob = self.out_bias()
+        self._out.set(take(tensors, self.out_tensor().name), None if ob is None else take(tensors, ob.name).float())
         self.bind_others(tensors, runtime)
 
     def linears(self) -> list:
@@ -75,6 +85,24 @@ class BranchMixer(Mixer):
             cache = cache[0] if cache else None
         self.attend(ctx, proj, 0, cache, o, 1.0)
         return self._out.forward(ctx, o, n)
+
+
+def _bias_specs(b) -> list[TensorSpec]:
+    return [s for s in (*b.in_biases(), b.out_bias()) if s is not None]
+
+
+def _in_bias(b, tensors):
+    """The biases of a branch's input matrices as float32 pieces in the order of the product's columns (zeros where a
+    matrix has none), or None if no matrix has one. Called before the matrices are taken out of the bag."""
+    specs, biases = b.in_tensors(), b.in_biases()
+    if all(x is None for x in biases):
+        return None
+    out = []
+    for spec, bias in zip(specs, biases):
+        w = tensors[spec.name]
+        out.append(take(tensors, bias.name).float() if bias is not None
+                   else torch.zeros(w.shape[0], dtype=torch.float32, device=w.device))
+    return out
 
 
 def _stacked(names, tensors, dim):
@@ -120,31 +148,48 @@ class ParallelMixer(Mixer):
 
     def tensor_specs(self) -> list[TensorSpec]:
         norms = [TensorSpec(n, (self.spec.hidden_size,), init="gain") for n in (self.spec.out_norms or ())]
-        return [s for b in self.branches for s in (*b.in_tensors(), b.out_tensor(), *b.other_tensors())] + norms
+        return [s for b in self.branches for s in (*b.in_tensors(), b.out_tensor(), *_bias_specs(b), *b.other_tensors())] + norms
 
     def bind(self, tensors, runtime) -> None:
         # every branch's columns start at a multiple of eight (rows of zeros between them), so that the
         # kernels which finish the product read them in 16-byte pieces
-        col, parts = 0, []
+        col, parts, biases = 0, [], []
         self.first_column = []
         for b in self.branches:
             self.first_column.append(col)
+            bias = _in_bias(b, tensors)
             mine = [take(tensors, s.name) for s in b.in_tensors()]
             rows = sum(t.shape[0] for t in mine)
             pad = -rows % COLUMN_ALIGN
             if pad and b is not self.branches[-1]:
                 mine.append(torch.zeros(pad, mine[0].shape[1], dtype=mine[0].dtype, device=mine[0].device))
                 rows += pad
+            biases.append(bias if bias is None else torch.cat(bias + [torch.zeros(rows - sum(x.numel() for x in bias),
+                                                                                  dtype=torch.float32, device=mine[0].device)]))
             parts += mine
             col += rows
         self.proj = Linear(self.spec.hidden_size, col, "mix.in")
-        self.proj.set(torch.cat(parts, dim=0))
+        bias = None
+        if any(x is not None for x in biases):  # one bias over all branches' columns, zero where a branch has none
+            rows = [*self.first_column[1:], col]
+            bias = torch.cat([x if x is not None else torch.zeros(rows[i] - self.first_column[i], dtype=torch.float32,
+                                                                  device=parts[0].device) for i, x in enumerate(biases)])
+        self.proj.set(torch.cat(parts, dim=0), bias)
         del parts, mine
         if self.spec.out_norms is None:
             self.out = Linear(self.inner, self.spec.hidden_size, "mix.out")
-            self.out.set(_stacked([b.out_tensor().name for b in self.branches], tensors, 1))
+            # the sum of the branches' output biases, each times its branch's factor
+            out_bias = None
+            for b, scale in zip(self.branches, self.spec.scales):
+                ob = b.out_bias()
+                if ob is not None:
+                    term = take(tensors, ob.name).float() * float(scale)
+                    out_bias = term if out_bias is None else out_bias + term
+            self.out.set(_stacked([b.out_tensor().name for b in self.branches], tensors, 1), out_bias)
         else:
             for i, (b, name) in enumerate(zip(self.branches, self.spec.out_norms)):
+                if b.out_bias() is not None:
+                    raise ValueError("parallel mixer: branches that are normed apart have no output bias")
                 lin = Linear(b.inner, self.spec.hidden_size, f"mix.out{i}")
                 lin.set(take(tensors, b.out_tensor().name))
                 self.outs.append(lin)

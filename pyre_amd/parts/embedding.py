@@ -21,8 +21,8 @@ class TokenEmbedding(Part):
         self.table = tensors[self.spec.name].contiguous()
 
     def forward(self, ctx, resid: torch.Tensor) -> None:
-        """resid[n] = float32(table[token n]): the residual stream starts here."""
-        ops.embed(self.table, ctx.tokens, resid)
+        """resid[n] = float32(table[token n]) * scale: the residual stream starts here."""
+        ops.embed(self.table, ctx.tokens, resid, self.spec.scale)
 
 
 class BigramEmbedding(Part):

@@ -92,7 +92,8 @@ def mid_ksplit(n_out: int, k: int, block_rows: int = 64, units: int = DEFAULT_UN
 LIBRARY_F32_ROLES = frozenset({"attn.qkv", "attn.out", "mix.in", "mix.out", "cattn.in", "cattn.out", "gla.in", "gla.out",
                                "glu.down", "tattn.qk", "tattn.out", "lattn.in", "lattn.out", "geglu.down", "moe.router",
                                "moe.down", "mix.out0", "mix.out1", "sattn.in", "sattn.out", "ret.in", "ret.out",
-                               "relu2.down", "gmoe.router", "gmoe.down"})
+                               "relu2.down", "gmoe.router", "gmoe.down", "wattn.in", "wattn.out", "gdr.in", "gdr.out",
+                               "stmoe.router", "stmoe.down", "side.gate", "side.proj"})
 
 
 def _is_bf16(ctx, lin, x) -> bool:

@@ -5,7 +5,7 @@ from __future__ import annotations
 import torch
 
 from pyre_amd.hip import ops
-from pyre_amd.parts.base import FeedForward, GroupedSoftmaxMoESpec, SigmoidMoESpec, TensorSpec, take
+from pyre_amd.parts.base import FeedForward, GroupedSoftmaxMoESpec, SigmoidMoESpec, SoftmaxTopKMoESpec, TensorSpec, take
 from pyre_amd.parts.linear import Linear
 
 
@@ -135,3 +135,75 @@ class GroupedSoftmaxMoE(FeedForward):
                 out = type(out)(full)
             ops.add_weighted_rows(out, h, gates, s.experts, s.identity, n)
         return out
+
+
+class SoftmaxTopKMoE(FeedForward):
+    """out = sum over the chosen experts e of w_e down_e(silu(gate_e h) * (up_e h)) + g down_s(silu(gate_s h) * (up_s h)):
+    the ``top`` experts of largest router logit z = R h + b, their weights the softmax over the chosen logits alone; the
+    shared expert s runs for every token, times g = sigmoid(sg . h).
+
+    The router's logits are a product of their own (float32 sums) whose last row is the shared expert's gate; one kernel
+    chooses, takes the softmax and writes a dense row of weights per token, the gate's sigmoid behind them. All experts'
+    gates and ways up, the shared one's behind them, are one product over [G_0; ..; G_E-1; G_s; U_0; ..; U_E-1; U_s], the
+    activation kernel gates, weights and zeroes, all ways down are one product over [D_0 | .. | D_E-1 | D_s], which sums
+    the weighted results as it goes. Every token streams through every expert's matrices."""
+
+    def __init__(self, spec: SoftmaxTopKMoESpec):
+        if not (0 < spec.top <= spec.experts <= ops.ROUTE_MAX_EXPERTS):
+            raise ValueError(f"mixture: {spec.top} of {spec.experts} experts is not a choice the routing kernel makes")
+        if spec.expert_size <= 0 or spec.shared_size < 0:
+            raise ValueError("mixture: bad expert sizes")
+        self.spec = spec
+        self.extra = 1 if spec.shared_size and spec.shared_gate else 0
+        self.inner = spec.experts * spec.expert_size + spec.shared_size
+        self.router = Linear(spec.hidden_size, spec.experts + self.extra, "stmoe.router")
+        self.gate_up = Linear(spec.hidden_size, 2 * self.inner, "stmoe.gate_up")
+        self.down = Linear(self.inner, spec.hidden_size, "stmoe.down")
+
+    def _experts(self) -> list[tuple[str, int]]:
+        s = self.spec
+        return [(f"{s.prefix}.e{i}", s.expert_size) for i in range(s.experts)] + \
+               ([(f"{s.prefix}.shared", s.shared_size)] if s.shared_size else [])
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        s = self.spec
+        specs = [TensorSpec(f"{s.prefix}.router", (s.experts, s.hidden_size))]
+        if s.router_bias:
+            specs.append(TensorSpec(f"{s.prefix}.router.b", (s.experts,)))
+        for p, ff in self._experts():
+            specs += [TensorSpec(f"{p}.gate", (ff, s.hidden_size)), TensorSpec(f"{p}.up", (ff, s.hidden_size)),
+                      TensorSpec(f"{p}.down", (s.hidden_size, ff))]
+        if self.extra:
+            specs.append(TensorSpec(f"{s.prefix}.shared.sg", (1, s.hidden_size)))
+        return specs
+
+    def bind(self, tensors, runtime) -> None:
+        s = self.spec
+        rows = [take(tensors, f"{s.prefix}.router")]
+        if self.extra:
+            rows.append(take(tensors, f"{s.prefix}.shared.sg").to(rows[0].dtype))
+        bias = None
+        if s.router_bias:
+            bias = take(tensors, f"{s.prefix}.router.b").float()
+            if self.extra:
+                bias = torch.cat([bias, torch.zeros(self.extra, dtype=torch.float32, device=bias.device)])
+        self.router.set(torch.cat(rows, dim=0) if len(rows) > 1 else rows[0], bias)
+        del rows
+        parts = [take(tensors, f"{p}.gate") for p, _ in self._experts()] + [take(tensors, f"{p}.up") for p, _ in self._experts()]
+        self.gate_up.set(torch.cat(parts, dim=0))
+        del parts
+        downs = [take(tensors, f"{p}.down") for p, _ in self._experts()]
+        self.down.set(torch.cat(downs, dim=1))
+        del downs
+
+    def linears(self) -> list:
+        return [self.router, self.gate_up, self.down]
+
+    def forward(self, ctx, h):
+        s, n, ws = self.spec, ctx.n_tokens, ctx.workspace
+        gates = ws.get("stmoe.gates", (n, s.experts + self.extra), torch.float32)
+        ops.route_topk(self.router.forward(ctx, h, n), gates, n, s.top, softmax=True, extra=self.extra)
+        act = ws.get("stmoe.act", (n, self.inner), ctx.dtype)
+        ops.expert_glu_act(self.gate_up.forward(ctx, h, n), gates, act, n, s.experts, s.expert_size, s.shared_size,
+                           s.experts if self.extra else -1)
+        return self.down.forward(ctx, act, n)

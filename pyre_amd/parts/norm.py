@@ -12,10 +12,13 @@ class RMSNorm(Norm):
         self.gain = None
 
     def tensor_specs(self) -> list[TensorSpec]:
-        return [TensorSpec(self.spec.tensor, (self.spec.hidden_size,), init="gain")]
+        return [TensorSpec(self.spec.tensor, (self.spec.hidden_size,), init="normal:0.1" if self.spec.one_plus else "gain")]
 
     def bind(self, tensors, runtime) -> None:
         self.gain = tensors[self.spec.tensor].contiguous()
+        if self.spec.one_plus:
+            # a weight stored around zero: the gain is one plus it, formed in float32 whatever the file's type
+            self.gain = (1.0 + self.gain.float()).contiguous()
 
     def forward(self, ctx, resid, delta, out, rows=None) -> None:
         if delta is not None and (delta.post is not None or delta.more is not None or delta.outer is not None
