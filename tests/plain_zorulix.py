@@ -203,19 +203,25 @@ def router_logits(w, p, h):
     return linear(w, f"{p}.router", h, True)
 
 
-def mixture(w, p, f, h):
+def mixture(w, p, f, h, calls=None):
     """The ``top`` experts of largest router logit, weighted by the softmax over their logits alone; a shared expert,
-    if the layer has one, for every token, times one sigmoid per token."""
+    if the layer has one, for every token, times one sigmoid per token. ``calls`` (a list) receives, per token, the gap
+    between the last logit that was chosen and the first that was not (inf if all were)."""
     E, top = f["router"]["experts"], f["router"]["top"]
     z = router_logits(w, p, h)
     out = torch.zeros_like(h)
+    gaps = []
     for t in range(h.shape[0]):
-        order = sorted(range(E), key=lambda e: (-float(z[t, e]), e))[:top]
+        ranked = sorted(range(E), key=lambda e: (-float(z[t, e]), e))
+        gaps.append(float(z[t, ranked[top - 1]] - z[t, ranked[top]]) if top < E else math.inf)
+        order = ranked[:top]
         weights = torch.softmax(z[t, order], dim=0)
         for e, a in zip(order, weights):
             out[t] += a * gated_unit(w, f"{p}.e{e}", h[t:t + 1])[0]
     if f.get("shared"):
         out = out + torch.sigmoid(h @ w[f"{p}.shared.sg"].T) * gated_unit(w, f"{p}.shared", h)
+    if calls is not None:
+        calls.append(gaps)
     return out
 
 
@@ -230,8 +236,9 @@ def token_side(w, p, x, ids, i, dim, eps):
 # ----------------------------------------------------------------------------- the model
 
 
-def forward(w, cfg, ids, return_hidden=False):
-    """Logits [T, vocab] of one sequence (float64); with ``return_hidden`` also the stream after every layer."""
+def forward(w, cfg, ids, return_hidden=False, calls=None):
+    """Logits [T, vocab] of one sequence (float64); with ``return_hidden`` also the stream after every layer. ``calls``:
+    see :func:`mixture` (one list per routed layer)."""
     eps = float(cfg["norm"]["eps"])
     ids = torch.as_tensor(list(ids), dtype=torch.long)
     x = w["embed"][ids] * float((cfg.get("embedding") or {}).get("scale", 1.0))
@@ -249,9 +256,19 @@ def forward(w, cfg, ids, return_hidden=False):
             raise ValueError(f"layer {i}: unknown type {layer['type']!r}")
         x = x + mixed
         if layer.get("mlp"):
-            x = x + mixture(w, f"{p}.mlp", layer["mlp"], one_plus_norm(x, w[f"{p}.norm2"], eps))
+            x = x + mixture(w, f"{p}.mlp", layer["mlp"], one_plus_norm(x, w[f"{p}.norm2"], eps), calls)
         if side:
             x = x + token_side(w, p, x, ids, i, side, eps)
         hidden.append(x.clone())
     logits = one_plus_norm(x, w["final.norm"], eps) @ w["head"].T
     return (logits, hidden) if return_hidden else logits
+
+
+def closest_call(w, cfg, ids):
+    """Per position the least gap, over the routed layers, by which the choice of experts was made (inf without any)."""
+    calls = []
+    forward(w, cfg, ids, calls=calls)
+    out = torch.full((len(ids),), math.inf, dtype=F)
+    for layer in calls:
+        out = torch.minimum(out, torch.tensor(layer, dtype=F))
+    return out

@@ -1,0 +1,698 @@
+"""The Zorulix design through the engine against the plain implementation (``plain_zorulix``): whole prompts layer by
+layer, prefill against token-by-token decoding, portions down to two tokens, mixed batches with pages and slots used
+again, long decoding past every window, keys made to stand out at the edges of a window and at page borders (also
+through the window of a layer that reads another's keys), a sink that decides the output, a state that must survive
+hundreds of tokens, each mixer alone, the kernels alone, greedy generation through the scheduler, and the programs as
+processes."""
+
+from __future__ import annotations
+
+import copy
+import json
+import math
+from dataclasses import dataclass
+from typing import ClassVar
+
+import numpy as np
+import pytest
+import torch
+
+import plain_zorulix as P
+import zorulix_models as M
+from helpers import cut, first_bad, random_ids, replay
+from pyre_amd.config.model import ModelConfig
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+#: bounds on max |difference| / max |logit| of a position: float32 against the float64 plain run (the recurrent branch
+#: subtracts what the state already holds from a token's value and divides its output by its root mean square, which
+#: takes a float32 run of a hundred tokens to a few 1e-5 where the differences cancel); bfloat16 loosely (the float32
+#: runs are the exact ones; heads of ten elements and weights drawn at 0.2 make 16-bit rows noisy)
+TOL = {"float32": 5e-5, "bfloat16": 1e-1}
+#: a 16-bit run is not compared where the plain router's choice hangs on less than this much of a logit (the logits are
+#: of the order of one, and a 16-bit run's are off by a few hundredths, now and then by a tenth and more)
+CLOSE_CALL = 0.25
+MODELS = {"small": (M.SMALL, 11), "ones": (M.ONES, 12), "wide": (M.WIDE, 13), "odd": (M.ODD, 14),
+          # for the 16-bit runs: one routed layer, the last, so that a close call spoils one position and not the rest
+          "small16": (M.routed_last(M.SMALL), 15), "odd16": (M.routed_last(M.ODD), 16)}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    from pyre_amd.registry import config_from_dict
+    from pyre_amd.weights import write_random_model
+
+    out = {}
+    for name, (raw, seed) in MODELS.items():
+        d = tmp_path_factory.mktemp("zorulix_" + name)
+        write_random_model(d, config_from_dict(raw), seed=seed, std=0.2, gain_std=0.2)
+        out[name] = (d, *P.read_folder(d))
+    return out
+
+
+def engine_of(folder, dtype, **kw):
+    from pyre_amd.config.engine import EngineConfig
+    from pyre_amd.engine.engine import Engine
+
+    args = dict(dtype=dtype, page_size=8, max_cached_tokens=1024, max_num_seqs=4, max_num_batched_tokens=512,
+                use_graphs=False)
+    args.update(kw)
+    return Engine.from_folder(folder, EngineConfig(**args))
+
+
+def plain_rows(cfg, w, ids):
+    return P.forward(w, cfg, ids).float()
+
+
+def whole(reqs):
+    return [([(r, ids, list(range(len(ids))))], [r]) for r, ids in reqs.items()]
+
+
+def in_portions(reqs, sizes):
+    steps = []
+    for r, ids in reqs.items():
+        pos, parts = 0, cut(len(ids), sizes)
+        for k, n in enumerate(parts):
+            steps.append(([(r, ids[pos:pos + n], list(range(n)))], [r] if k == len(parts) - 1 else []))
+            pos += n
+    return steps
+
+
+def one_by_one(reqs, first):
+    steps = []
+    for r, ids in reqs.items():
+        steps.append(([(r, ids[:first], list(range(first)))], []))
+        steps += [([(r, [ids[t]], [0])], [r] if t == len(ids) - 1 else []) for t in range(first, len(ids))]
+    return steps
+
+
+def assert_close(got, want, tol, calls=None):
+    """``calls``: request -> :func:`plain_zorulix.closest_call` of its tokens (16-bit runs)."""
+    if calls is not None:
+        # A sequence's first token leaves one term in the recurrent state, and the unit norm of the head's output turns
+        # it into sign(q . k) u / rms(u): where q . k happens to be near zero, 16-bit rounding decides the sign, and the
+        # row is no measure of the engine. The 32-bit runs compare that position like every other.
+        got = {(r, pos): row for (r, pos), row in got.items() if pos != 0 and float(calls[r][pos]) >= CLOSE_CALL}
+    bad, worst = first_bad(got, want, tol)
+    assert bad is None, bad
+    return worst
+
+
+def calls_of(cfg, w, reqs, dtype):
+    return {r: P.closest_call(w, cfg, ids) for r, ids in reqs.items()} if dtype == "bfloat16" else None
+
+
+def all_given_back(eng):
+    eng.cache.check_invariants()
+    return all(g.allocator.num_used == 0 for g in eng.cache.page_groups) and eng.cache.slots.num_used == 0
+
+
+# ----------------------------------------------------------------------------- whole prompts, layer by layer
+
+
+@pytest.mark.parametrize("name", ["small", "ones", "wide", "odd"])
+def test_every_layer_of_a_whole_prompt(name, folders):
+    from pyre_amd.engine.batch import Entry
+
+    folder, cfg, w = folders[name]
+    ids = random_ids(cfg["vocab"], 75, seed=3)
+    want, layers = P.forward(w, cfg, ids, return_hidden=True)
+    eng = engine_of(folder, "float32")
+    seen = {}
+    got = eng.step([Entry("a", ids, list(range(len(ids))))], tap=lambda pos, rows: seen.__setitem__(pos, rows.double().cpu()))
+    for pos, ref in enumerate(layers):
+        d = float((seen[pos] - ref).abs().max() / ref.abs().max())
+        assert d <= TOL["float32"], f"layer {pos}: {d:.2e}"
+    d = float((got.double().cpu() - want).abs().max() / want.abs().max())
+    assert d <= TOL["float32"], d
+
+
+# (the model of single heads of two and three elements runs in float32 only: in 16 bits its logits are mostly rounding)
+@pytest.mark.parametrize("name,dtype,page", [("small", "float32", 8), ("small16", "bfloat16", 16), ("ones", "float32", 4),
+                                             ("wide", "float32", 16), ("odd", "float32", 8), ("odd16", "bfloat16", 16)])
+def test_prefill_decode_and_portions_agree_with_plain(name, dtype, page, folders):
+    folder, cfg, w = folders[name]
+    reqs = {r: random_ids(cfg["vocab"], n, seed=n) for r, n in (("a", 90), ("b", 1), ("c", 37))}
+    want = {r: plain_rows(cfg, w, ids) for r, ids in reqs.items()}
+    calls = calls_of(cfg, w, reqs, dtype)
+    eng = engine_of(folder, dtype, page_size=page)
+    assert_close(replay(eng, whole(reqs)), want, TOL[dtype], calls)
+    # most of the prompt, then token by token: the windows pass over decoded tokens
+    tail = {r: ids for r, ids in reqs.items() if len(ids) > 1}
+    assert_close(replay(eng, one_by_one(tail, 6)), want, TOL[dtype], calls)
+    # the first tokens of a sequence one by one from the very start: the convolution's zeros, the empty state
+    assert_close(replay(eng, one_by_one({"c": reqs["c"][:12]}, 1)), want, TOL[dtype], calls)
+    for sizes in ([2], [3, 2, 17, 2, 31, 5], [64, 2, 9], [7, 1, 1, 24]):
+        assert_close(replay(eng, in_portions(tail, sizes)), want, TOL[dtype], calls)
+    assert all_given_back(eng)
+
+
+@pytest.mark.parametrize("name,dtype,poison", [("small", "float32", True), ("wide", "float32", True), ("small16", "bfloat16", False),
+                                               ("ones", "float32", True), ("odd", "float32", True)])
+def test_mixed_batches_with_pages_and_slots_used_again(name, dtype, poison, folders):
+    folder, cfg, w = folders[name]
+    reqs = {r: random_ids(cfg["vocab"], n, seed=7 * n) for r, n in (("a", 61), ("b", 9), ("c", 100), ("d", 33), ("e", 2), ("f", 47))}
+    want = {r: plain_rows(cfg, w, ids) for r, ids in reqs.items()}
+    # three slots, a pool that holds three of the requests at most: everything is used again
+    eng = engine_of(folder, dtype, max_num_seqs=3, max_cached_tokens=232, debug_poison=poison)
+    fed = {r: 0 for r in reqs}
+    live, waiting, steps, k = [], list(reqs), [], 0
+    while live or waiting:
+        while waiting and len(live) < 3:
+            live.append(waiting.pop(0))
+        entries, end = [], []
+        for r in live:
+            n = min([5, 1, 13, 2, 1, 40, 1][k % 7], len(reqs[r]) - fed[r])
+            k += 1
+            entries.append((r, reqs[r][fed[r]:fed[r] + n], list(range(n))))
+            fed[r] += n
+            if fed[r] == len(reqs[r]):
+                end.append(r)
+        steps.append((entries, end))
+        live = [r for r in live if r not in end]
+    got = replay(eng, steps)
+    assert_close(got, want, TOL[dtype], calls_of(cfg, w, reqs, dtype))
+    assert all_given_back(eng)
+    # every request alone gives the same rows, beyond rounding: batch-mates, pages and slots do not matter
+    alone = engine_of(folder, dtype)
+    for r in ("a", "d"):
+        single = replay(alone, whole({r: reqs[r]}))
+        for pos in range(len(reqs[r])):
+            d = float((single[(r, pos)] - got[(r, pos)]).abs().max() / want[r][pos].abs().max())
+            assert d <= (TOL[dtype] if dtype == "float32" else 2 * TOL[dtype]), (r, pos, d)
+
+
+def test_long_decoding_in_a_pool_that_only_windows_make_fit(folders):
+    """260 tokens one by one through a model whose layers all have windows (one of them reading another's pages through a
+    wider window than the owner's): the pages go back as the windows pass, so a pool of 80 tokens is enough; the
+    recurrent branch and the convolution carry on all the while."""
+    folder, cfg, w = folders["small"]
+    ids = random_ids(cfg["vocab"], 260, seed=1)
+    want = {"a": plain_rows(cfg, w, ids)}
+    eng = engine_of(folder, "float32", page_size=8, max_cached_tokens=80, max_model_len=512, debug_poison=True)
+    assert_close(replay(eng, one_by_one({"a": ids}, 2)), want, TOL["float32"])
+    assert all(g.allocator.num_used == 0 for g in eng.cache.page_groups)
+
+
+_made = {}
+
+
+def _folder_of(raw, seed, tensors=None, config=None):
+    """A model folder for ``raw`` (cached by its text); ``tensors(state)`` may change the drawn weights."""
+    import tempfile
+
+    from safetensors.torch import save_file
+
+    from pyre_amd.registry import config_from_dict
+    from pyre_amd.weights import model_tensor_specs, random_state
+
+    key = (json.dumps(raw, sort_keys=True), seed, tensors)
+    if key not in _made:
+        d = tempfile.mkdtemp(prefix="zorulix_")
+        cfg = config_from_dict(raw) if config is None else config
+        cfg.save(d)
+        state = random_state(model_tensor_specs(cfg), seed, 0.2, 0.2)
+        if tensors is not None:
+            tensors(state)
+        save_file({k: v.contiguous() for k, v in state.items()}, d + "/model.safetensors")
+        _made[key] = (d, *P.read_folder(d))
+    return _made[key]
+
+
+# ----------------------------------------------------------------------------- keys made to stand out
+
+
+#: two attention layers without rotation, so that a token's key is the same wherever it stands: a window of 12 tokens on
+#: pages of 8, read again by a second layer through a window of 19; a large scale makes the softmax sharp
+EDGE = M.model(53, 32, [M.attention(M.attn(2, 1, 16, 8, 6.0, window=12), M.moe(3, 1, 8)),
+                        M.attention(M.attn(2, 1, 16, 8, 6.0, window=19, kv_from=0))], eps=1e-5, scale=2.0, side=2)
+
+
+def _keys_like_queries(state):
+    # Queries and keys read the first half of a row, values the second; keys are made by the first head's query matrix.
+    # Token 51 shares the first half of its row with token 52: its key points where 52's query points, and its value is
+    # another. A query of token 52 then gives its weight to itself and to an earlier 51, half each (the norm over the
+    # projection gives both keys one length), so that whether the 51 is seen decides its output; the sink's one is
+    # small beside the exponentials of these scores.
+    for p in ("l0.mix", "l1.mix"):
+        q = state[f"{p}.q"]
+        q[:, 16:] = 0
+        state[f"{p}.q.b"].zero_()
+        state[f"{p}.q.norm"].fill_(1.0)
+    state["l0.mix.k"] = state["l0.mix.q"][:16].clone()
+    state["l1.mix.q"] = state["l0.mix.q"].clone()
+    state["l0.mix.k.b"].zero_()
+    state["l0.mix.k.norm"].fill_(1.0)
+    state["l0.mix.v"][:, :16] = 0
+    state["embed"][51, :16] = state["embed"][52, :16]
+    # the second layer's rows must still tell the first half of 51's and 52's rows alike: what the first layer adds is small
+    for n in ("l0.mix.o", "l0.side.proj", "l0.side.norm"):
+        state[n] *= 0.01
+    for e in range(3):
+        state[f"l0.mlp.e{e}.down"] *= 0.01
+
+
+@pytest.mark.parametrize("layer,window", [(0, 12), (1, 19)])
+def test_a_key_just_inside_and_just_outside_the_window(layer, window):
+    """The second case looks through the window of the layer that reads the first one's pages: keys that the owner's
+    window has passed must still be there for it."""
+    raw = copy.deepcopy(EDGE)
+    if layer == 0:
+        raw["layers"] = raw["layers"][:1]
+    else:
+        raw["layers"][0]["mixer"]["scale"] = 0.01    # the first layer spreads its weight: it decides nothing
+    folder, cfg, w = _folder_of(raw, 31, _keys_like_queries if layer == 1 else _keys_one_layer)
+    T, twin = 52, 51
+    eng = engine_of(folder, "float32", page_size=8)
+    base = [1 + (i % 50) for i in range(60)]           # no token twice within 50 positions; 51 and 52 appear nowhere
+    cases = {"inside": (40, 40 - (window - 1)), "outside": (40, 40 - window), "page_border": (47, 40), "far": (57, 9),
+             "next_to_it": (40, 39)}
+    reqs = {}
+    for name, (i, j) in cases.items():
+        ids = list(base)
+        ids[i], ids[j] = T, twin
+        reqs[name] = ids
+    want = {r: plain_rows(cfg, w, ids) for r, ids in reqs.items()}
+    # the construction works: whether the twin is seen decides the logits at the query
+    seen = float((want["inside"][40] - want["outside"][40]).abs().max() / want["inside"][40].abs().max())
+    assert seen > 500 * TOL["float32"], seen
+    for steps in (whole(reqs), one_by_one(reqs, 30), in_portions(reqs, [39, 2, 5]), in_portions(reqs, [2, 3])):
+        assert_close(replay(eng, steps), want, TOL["float32"])
+    eng16 = engine_of(folder, "bfloat16", page_size=16)
+    for steps in (whole(reqs), one_by_one(reqs, 35)):
+        assert_close(replay(eng16, steps), want, TOL["bfloat16"], {r: [1.0] * len(ids) for r, ids in reqs.items()})
+
+
+def _keys_one_layer(state):
+    q = state["l0.mix.q"]
+    q[:, 16:] = 0
+    state["l0.mix.q.b"].zero_(), state["l0.mix.k.b"].zero_()
+    state["l0.mix.q.norm"].fill_(1.0), state["l0.mix.k.norm"].fill_(1.0)
+    state["l0.mix.k"] = q[:16].clone()
+    state["l0.mix.v"][:, :16] = 0
+    state["embed"][51, :16] = state["embed"][52, :16]
+
+
+def test_a_sink_that_decides_the_output():
+    """With small scores the sink's one is a large share of every denominator: leaving it out, or counting it twice,
+    would move the logits far beyond rounding."""
+    raw = copy.deepcopy(EDGE)
+    raw["layers"][0]["mixer"]["scale"] = 0.05
+    raw["layers"][1]["mixer"]["scale"] = 0.02
+    folder, cfg, w = _folder_of(raw, 33)
+    reqs = {"a": random_ids(cfg["vocab"], 50, seed=4), "b": random_ids(cfg["vocab"], 3, seed=5)}
+    want = {r: plain_rows(cfg, w, ids) for r, ids in reqs.items()}
+    real = P.attention_mixer
+    try:
+        P.attention_mixer = lambda *a, **k: real(*a, **{**k, "sink": False})
+        moved = float((plain_rows(cfg, w, reqs["a"]) - want["a"]).abs().max() / want["a"].abs().max())
+    finally:
+        P.attention_mixer = real
+    assert moved > 500 * TOL["float32"], moved
+    eng = engine_of(folder, "float32", page_size=8)
+    for steps in (whole(reqs), one_by_one(reqs, 2), in_portions(reqs, [2, 7])):
+        assert_close(replay(eng, steps), want, TOL["float32"])
+
+
+def test_a_state_that_has_to_last():
+    """Decays close to one: the first tokens reach the last logits through the recurrent state alone (the window is 12
+    tokens, the changed token is the fourth)."""
+    raw = M.model(53, 32, [M.parallel(M.attn(2, 1, 16, 8, 0.3, window=12, rot=M.rot(100.0, 8)), M.delta(4, 2, 8, 8, 3), 0.6, 1.4,
+                                      M.moe(3, 2, 8, shared=4))], eps=1e-5, scale=2.0, side=3)
+
+    def slow(state):
+        state["l0.mix.right.A_log"].fill_(-7.0)
+
+    folder, cfg, w = _folder_of(raw, 32, slow)
+    ids = random_ids(cfg["vocab"], 300, seed=9)
+    other = list(ids)
+    other[3] = (ids[3] + 1) % cfg["vocab"]
+    want = {"a": plain_rows(cfg, w, ids), "b": plain_rows(cfg, w, other)}
+    moved = float((want["a"][-1] - want["b"][-1]).abs().max() / want["a"][-1].abs().max())
+    assert moved > 1e-3, moved
+    eng = engine_of(folder, "float32", page_size=16, max_cached_tokens=640)
+    reqs = {"a": ids, "b": other}
+    assert_close(replay(eng, whole(reqs)), want, TOL["float32"])
+    assert_close(replay(eng, in_portions(reqs, [64, 2, 31, 100, 3])), want, TOL["float32"])
+    assert_close(replay(eng, one_by_one({"a": ids}, 30)), want, TOL["float32"])
+
+
+# ----------------------------------------------------------------------------- each mechanism alone
+
+
+@dataclass(frozen=True)
+class OneMixerConfig(ModelConfig):
+    """A model of pre-norm layers whose mixer is a single one: 'attention', 'left' or 'right' of the design, without
+    feed-forward and without the token side input."""
+
+    raw: dict
+    architecture: ClassVar[str] = "ToyOneMixer"
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(raw)
+
+    def to_dict(self):
+        return self.raw
+
+    def save(self, folder):
+        import pathlib
+        pathlib.Path(folder, "config.json").write_text(json.dumps(self.raw))
+
+    def __hash__(self):
+        return id(self)
+
+
+def _build_one_mixer(cfg):
+    from pyre_amd.config.zorulix import AttentionConfig, DeltaRuleConfig
+    from pyre_amd.models.zorulix import _position
+    from pyre_amd.parts.base import (BlockSpec, EmbeddingSpec, GatedDeltaRuleSpec, LayerCall, LMHeadSpec, ModelSpec,
+                                     RMSNormSpec, WindowAttentionSpec)
+
+    raw = cfg.raw
+    width, eps = raw["width"], raw["norm"]["eps"]
+    layers = []
+    for i, layer in enumerate(raw["layers"]):
+        p = f"l{i}.mix"
+        if layer["type"] == "right":
+            r = DeltaRuleConfig.from_dict(layer["mixer"], "right")
+            mixer = GatedDeltaRuleSpec(width, r.heads, r.kv_heads, r.dim, r.vdim, r.conv, p, norm_eps=eps)
+        else:
+            a = AttentionConfig.from_dict(layer["mixer"], "left")
+            whole = layer["type"] == "attention"
+            mixer = WindowAttentionSpec(width, a.heads, a.kv_heads, a.dim, a.vdim, a.scale, _position(a), p, window=a.window,
+                                        out_bias=not whole, wide_norm=whole, norm_eps=eps, sink="zero" if whole else "none")
+        layers.append(BlockSpec(mixer, RMSNormSpec(width, eps, "", name=f"l{i}.norm1", one_plus=True), None, None))
+    return ModelSpec(width, raw["vocab"], 0, EmbeddingSpec(raw["vocab"], width, name="embed"), tuple(layers),
+                     tuple(LayerCall(i) for i in range(len(layers))), RMSNormSpec(width, eps, "", name="final.norm", one_plus=True),
+                     LMHeadSpec(raw["vocab"], width, name="head"))
+
+
+def _plain_one_mixer(w, raw, ids):
+    eps = raw["norm"]["eps"]
+    x = w["embed"][torch.as_tensor(ids)]
+    for i, layer in enumerate(raw["layers"]):
+        h = P.one_plus_norm(x, w[f"l{i}.norm1"], eps)
+        if layer["type"] == "right":
+            x = x + P.delta_rule_mixer(w, f"l{i}.mix", layer["mixer"], h, eps)
+        else:
+            whole = layer["type"] == "attention"
+            x = x + P.attention_mixer(w, f"l{i}.mix", layer["mixer"], h, eps, sink=whole, whole_norm=whole, out_bias=not whole)[0]
+    return (P.one_plus_norm(x, w["final.norm"], eps) @ w["head"].T).float()
+
+
+@pytest.mark.parametrize("kind", ["attention", "left", "right"])
+def test_each_mixer_alone(kind, tmp_path):
+    from pyre_amd.registry import register_architecture, unregister_architecture
+    from pyre_amd.weights import write_random_model
+
+    mixers = {"attention": [M.attn(4, 2, 24, 16, 0.5, window=20, rot=M.rot(100.0, 10)), M.attn(5, 1, 7, 9, 0.8),
+                            M.attn(2, 1, 12, 8, 0.6, window=5, rot=M.rot(10.0, 12))],
+              "left": [M.attn(4, 4, 10, 6, 0.4, window=9, rot=M.rot(50.0, 10, (3.0, 40, 6.0, 0.8))), M.attn(3, 1, 132, 12, 0.1, window=31)],
+              # (nine taps: more than the first portions are long)
+              "right": [M.delta(2, 2, 16, 24, 3), M.delta(6, 3, 33, 7, 1), M.delta(2, 1, 5, 70, 9)]}[kind]
+    raw = {"architectures": ["ToyOneMixer"], "vocab": 71, "width": 40, "norm": {"eps": 1e-5},
+           "layers": [{"type": kind, "mixer": m, "mlp": None} for m in mixers]}
+    register_architecture(OneMixerConfig.architecture, OneMixerConfig, _build_one_mixer)
+    try:
+        write_random_model(tmp_path, OneMixerConfig(raw), seed=41, std=0.2, gain_std=0.2)
+        _, w = P.read_folder(tmp_path)
+        reqs = {r: random_ids(71, n, seed=n) for r, n in (("a", 70), ("b", 19))}
+        want = {r: _plain_one_mixer(w, raw, ids) for r, ids in reqs.items()}
+        eng = engine_of(tmp_path, "float32")
+        kinds = [[type(s).__name__ for s in c] for c in eng.model.cache_specs()]
+        assert kinds == ([["PagedCacheSpec"]] * len(mixers) if kind != "right" else
+                         [["StateCacheSpec", "StateCacheSpec"], ["StateCacheSpec"], ["StateCacheSpec", "StateCacheSpec"]])
+        assert_close(replay(eng, whole(reqs)), want, TOL["float32"])
+        assert_close(replay(eng, in_portions(reqs, [5, 2, 30])), want, TOL["float32"])
+        assert_close(replay(eng, one_by_one(reqs, 4)), want, TOL["float32"])
+    finally:
+        unregister_architecture(OneMixerConfig.architecture)
+
+
+@pytest.mark.parametrize("nq,nkv,dk,dv,rot", [(4, 2, 16, 8, 8), (3, 0, 10, 6, 10), (2, 2, 136, 4, 0), (1, 1, 6, 5, 2)])
+def test_the_kernel_that_norms_a_whole_projection(nq, nkv, dk, dv, rot):
+    """The product's partial sums and bias, the norm over all query (and all key) columns, the turn of part of a head,
+    the stores to rows and pages; a layer without keys of its own has queries alone."""
+    from pyre_amd.hip import ops
+    from pyre_amd.parts.rotary import rotary_tables
+
+    g = torch.Generator().manual_seed(nq * dk)
+    n, page, col0 = 11, 4, 8
+    width = col0 + (nq + nkv) * dk + nkv * dv + 3
+    parts = torch.randn(2, n, width, generator=g)
+    bias = torch.randn(width, generator=g)
+    qg, kg = 1 + 0.3 * torch.randn(nq * dk, generator=g), 1 + 0.3 * torch.randn(max(nkv, 1) * dk, generator=g)
+    positions = torch.arange(5, 5 + n, dtype=torch.int32)
+    cos, sin = rotary_tables(rot, 100.0, 32, exact=True) if rot else (None, None)
+    u = (parts.double().sum(0) + bias.double())[:, col0:]
+    rows = {"q": u[:, :nq * dk], "k": u[:, nq * dk:(nq + nkv) * dk]}
+    want = {}
+    for name, gain, heads in (("q", qg, nq), ("k", kg, nkv)):
+        if not heads:
+            continue
+        x = (P.unit_rms(rows[name], 1e-5) * gain.double()).reshape(n, heads, dk)
+        if rot:
+            y = x.clone()
+            half = rot // 2
+            for t in range(n):
+                c, s = cos[positions[t]].double(), sin[positions[t]].double()
+                y[t, :, :half] = x[t, :, :half] * c - x[t, :, half:rot] * s
+                y[t, :, half:rot] = x[t, :, half:rot] * c + x[t, :, :half] * s
+            x = y
+        want[name] = x
+    for dtype, tol in ((torch.float32, 2e-6), (torch.bfloat16, 1e-2)):
+        q = torch.empty(n, nq * dk, device=DEV, dtype=dtype)
+        kc = torch.zeros(8, max(nkv, 1), page, dk, device=DEV, dtype=dtype) if nkv else None
+        vc = torch.zeros(8, max(nkv, 1), page, dv, device=DEV, dtype=dtype) if nkv else None
+        slots = torch.tensor([4 * 3 + 1 + t for t in range(n)], dtype=torch.int32, device=DEV)
+        ops.wide_norm_qkv_write(ops.Partials(parts.to(DEV), bias.to(DEV)), col0, qg.to(DEV), kg.to(DEV) if nkv else None, 1e-5,
+                                cos.to(DEV) if rot else None, sin.to(DEV) if rot else None, rot, positions.to(DEV), q, kc, vc,
+                                slots if nkv else None, n, nq, nkv, dk, dv, page)
+        assert float((q.cpu().double().reshape(n, nq, dk) - want["q"]).abs().max()) < tol * float(want["q"].abs().max())
+        if nkv:
+            for t in range(n):
+                s = int(slots[t])
+                kt, vt = kc[s // page, :, s % page].cpu().double(), vc[s // page, :, s % page].cpu().double()
+                assert float((kt - want["k"][t]).abs().max()) < tol * float(want["k"].abs().max())
+                vw = u[t, (nq + nkv) * dk:(nq + nkv) * dk + nkv * dv].reshape(nkv, dv)
+                assert float((vt - vw).abs().max()) < tol * float(vw.abs().max())
+
+
+@pytest.mark.parametrize("H,G,dk,dv", [(2, 1, 8, 8), (3, 3, 33, 70), (4, 2, 130, 5), (1, 1, 1, 1)])
+def test_the_delta_rule_kernels(H, G, dk, dv):
+    """The recurrence alone, from a state that is not empty, over requests of unequal lengths in one launch; then its
+    finishing kernel."""
+    from pyre_amd.hip import ops
+
+    g = torch.Generator().manual_seed(H * dk + dv)
+    lens = [7, 1, 12]
+    n, width = sum(lens), ops.gdr_row_width(H, G, dk, dv)
+    x = torch.randn(n, width, generator=g)
+    a0, v0, g0, b0 = 2 * G * dk, 2 * G * dk + H * dk, 2 * G * dk + H * dk + H * dv, 2 * G * dk + H * dk + 2 * H * dv
+    x[:, a0:v0] = torch.rand(n, H * dk, generator=g) * 0.5 + 0.5            # decays
+    x[:, b0:] = torch.rand(n, H, generator=g)                               # betas
+    x[:, g0:b0] = torch.rand(n, H * dv, generator=g)                        # gates
+    state = torch.randn(5, H, dk, dv, generator=g)
+    slots = [3, 0, 4]
+    want_state, want_o = state.double().clone(), torch.zeros(n, H, dv, dtype=torch.float64)
+    t0 = 0
+    for s, ln in zip(slots, lens):
+        for t in range(t0, t0 + ln):
+            xr = x[t].double()
+            for hd in range(H):
+                gq = hd // (H // G)
+                q, k = xr[gq * dk:(gq + 1) * dk], xr[G * dk + gq * dk:G * dk + (gq + 1) * dk]
+                S = want_state[s, hd] * xr[a0 + hd * dk:a0 + (hd + 1) * dk].unsqueeze(1)
+                uu = xr[b0 + hd] * (xr[v0 + hd * dv:v0 + (hd + 1) * dv] - S.T @ k)
+                S = S + torch.outer(k, uu)
+                want_state[s, hd] = S
+                want_o[t, hd] = S.T @ q
+        t0 += ln
+    st, o = state.to(DEV), torch.empty(n, H * dv, device=DEV)
+    q_start = torch.tensor([0, 7, 8, 20], dtype=torch.int32, device=DEV)
+    ops.gdr_scan(x.to(DEV), st, o, q_start, torch.tensor(slots, dtype=torch.int32, device=DEV), 3, H, G, dk, dv)
+    scale = float(want_o.abs().max())
+    assert float((o.cpu().double().reshape(n, H, dv) - want_o).abs().max()) < 2e-5 * scale
+    assert float((st.cpu().double() - want_state).abs().max()) < 2e-5 * float(want_state.abs().max())
+    assert torch.equal(st[[1, 2]].cpu(), state[[1, 2]])
+    gain = 1 + 0.2 * torch.randn(dv, generator=g)
+    want = P.unit_rms(want_o, 1e-4) * gain.double() * x[:, g0:b0].double().reshape(n, H, dv) * 0.7
+    for dtype, tol in ((torch.float32, 3e-5), (torch.bfloat16, 1e-2)):
+        out = torch.zeros(n, H * dv + 3, device=DEV, dtype=dtype)
+        ops.gdr_finish(o, x.to(DEV), gain.to(dtype).to(DEV), 1e-4, 0.7, out[:, 3:], n, H, G, dk, dv)
+        ref = P.unit_rms(want_o, 1e-4) * gain.to(dtype).double() * x[:, g0:b0].double().reshape(n, H, dv) * 0.7
+        assert float((out[:, 3:].cpu().double().reshape(n, H, dv) - ref).abs().max()) < tol * float(want.abs().max())
+
+
+@pytest.mark.parametrize("experts,top,extra", [(6, 2, 1), (10, 3, 0), (8, 8, 1), (130, 5, 1), (3, 1, 0), (1, 1, 1)])
+def test_the_routing_kernel_with_a_softmax_over_the_chosen(experts, top, extra):
+    from pyre_amd.hip import ops
+
+    g = torch.Generator().manual_seed(experts)
+    n = 40
+    z = torch.randn(2, n, experts + extra, generator=g) * 2
+    z[:, 5] = z[:, 5].round()            # rows with equal logits: the lower index wins
+    z[:, 6] = 0.0
+    bias = torch.randn(experts + extra, generator=g)
+    gates = torch.full((n, experts + extra), -1.0, device=DEV)
+    ops.route_topk(ops.Partials(z.to(DEV), bias.to(DEV)), gates, n, top, softmax=True, extra=extra)
+    gates = gates.cpu().double()
+    for t in range(n):
+        zt = z[:, t].double().sum(0) + bias.double()
+        order = sorted(range(experts), key=lambda e: (-float(zt[e]), e))[:top]
+        want = torch.zeros(experts + extra, dtype=torch.float64)
+        want[order] = torch.softmax(zt[order], 0)
+        if extra:
+            want[experts:] = torch.sigmoid(zt[experts:])
+        if top < experts and abs(float(zt[order[-1]] - sorted(zt[:experts].tolist(), reverse=True)[top])) < 1e-6 and t not in (5, 6):
+            continue
+        assert float((gates[t] - want).abs().max()) < 1e-6, (t, order, gates[t].nonzero().flatten().tolist())
+    # the sigmoid form still answers as before
+    ops.route_topk(ops.Partials(z[:, :, :experts].contiguous().to(DEV)), gates_dev := torch.empty(n, experts, device=DEV), n, top)
+    s = torch.sigmoid(z[:, 0, :experts].double().sum(0))
+    order = sorted(range(experts), key=lambda e: (-float(s[e]), e))[:top]
+    want = torch.zeros(experts, dtype=torch.float64)
+    want[order] = s[order] / (s[order].sum() + 1e-20)
+    assert float((gates_dev[0].cpu().double() - want).abs().max()) < 1e-6
+
+
+def test_the_experts_activation_with_a_shared_expert_and_the_token_side_gate():
+    from pyre_amd.hip import ops
+
+    g = torch.Generator().manual_seed(8)
+    for n, experts, ff, shared, gated in ((7, 3, 10, 6, True), (5, 2, 8, 12, False), (4, 4, 8, 0, False), (3, 1, 3, 1, True)):
+        width = experts * ff + shared
+        gu = torch.randn(2, n, 2 * width, generator=g)
+        gates = torch.rand(n, experts + 1, generator=g)
+        gates[:, :experts][gates[:, :experts] < 0.4] = 0.0
+        total = gu.double().sum(0)
+        weights = torch.cat([gates.double()[:, :experts].repeat_interleave(ff, 1),
+                             (gates.double()[:, experts:] if gated else torch.ones(n, 1, dtype=torch.float64)).expand(n, shared)], 1)
+        want = weights * P.silu(total[:, :width]) * total[:, width:]
+        for dtype, tol in ((torch.float32, 1e-6), (torch.bfloat16, 1e-2)):
+            out = torch.empty(n, width, device=DEV, dtype=dtype)
+            ops.expert_glu_act(ops.Partials(gu.to(DEV)), gates.to(DEV), out, n, experts, ff, shared, experts if gated else -1)
+            assert float((out.cpu().double() - want).abs().max()) < tol * float(want.abs().max())
+    n, dim, tw, first = 9, 5, 17, 10
+    z, bias = torch.randn(3, n, dim, generator=g) * 2, torch.randn(dim, generator=g)
+    table = torch.randn(20, tw, generator=g)
+    ids = torch.randint(0, 20, (n,), generator=g, dtype=torch.int32)
+    want = P.gelu_tanh(z.double().sum(0) + bias.double()) * table.double()[ids.long(), first:first + dim]
+    out = torch.empty(n, dim, device=DEV)
+    ops.token_side_gate(ops.Partials(z.to(DEV), bias.to(DEV)), table.to(DEV), first, ids.to(DEV), out, n)
+    assert float((out.cpu().double() - want).abs().max()) < 2e-6 * float(want.abs().max())
+
+
+def test_stretched_frequencies_against_their_definition():
+    from pyre_amd.parts.rotary import rotary_tables
+
+    for r in (M.rot(3000.0, 16, (4.0, 64, 8.0, 0.5)), M.rot(50000.0, 64, (2.0, 1024, 32.0, 1.0)), M.rot(100.0, 6, (16.0, 8, 2.0, 1.5)),
+              M.rot(10.0, 4)):
+        f, mag = P.frequencies(r)
+        sc = r.get("scaling")
+        cos, sin = rotary_tables(r["dims"], r["base"], 300, exact=True,
+                                 scaling=None if not sc else (sc["factor"], sc["original"], sc["fast"], sc["slow"]))
+        for p in (0, 1, 17, 299):
+            for i, fi in enumerate(f):
+                assert abs(float(cos[p, i]) - math.cos(p * fi) * mag) < 2e-6 and abs(float(sin[p, i]) - math.sin(p * fi) * mag) < 2e-6
+
+
+# ----------------------------------------------------------------------------- the entry points
+
+
+@pytest.mark.parametrize("graphs", [False, True])
+def test_greedy_generation_through_the_scheduler(graphs, folders):
+    """The scheduler runs one step ahead, its tokens fed on the device: the token side input reads them there. With
+    graphs the decode steps are captured and replayed."""
+    from pyre_amd.api import generate, load_model
+
+    folder, cfg, w = folders["small"]
+    prompts = [random_ids(cfg["vocab"], n, seed=n + 1) for n in (1, 9, 40, 23)]
+    eng, _ = load_model(str(folder), device=DEV, dtype="float32", page_size=8, max_cached_tokens=1024, max_num_seqs=4,
+                        max_num_batched_tokens=64, prefill_chunk=16, use_graphs=graphs)
+    got = generate(eng, prompts, max_new_tokens=30)
+    for p, g in zip(prompts, got):
+        assert len(g) == 30
+        ids = list(p)
+        for k, tok in enumerate(g):
+            row = P.forward(w, cfg, ids)[-1]
+            twin = int(row.argmax())
+            if twin != tok:
+                margin = float((row[twin] - row[tok]) / row.abs().max())
+                assert margin < TOL["float32"], f"token {k} is {tok}, plainly {twin} (margin {margin:.2e})"
+            ids.append(tok)
+    assert all_given_back(eng)
+    if graphs:
+        assert eng.graph_replays > 0
+
+
+def test_the_generate_program_as_a_process(folders, tmp_path):
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    folder, cfg, w = folders["odd"]
+    root = Path(__file__).resolve().parent.parent
+    out = tmp_path / "res.json"
+    proc = subprocess.run([sys.executable, str(root / "bin" / "pyre_generate"), "--model", str(folder), "--dtype", "float32",
+                           "--prompt-ids", "7,3,3,41,9,50,5", "--prompt-ids", "11", "--tokens", "12", "--num-blocks", "32",
+                           "--max-batch", "2", "--out", str(out)], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    res = json.loads(out.read_text())
+    assert res["dtype"] == "float32" and [len(g) for g in res["generated"]] == [12, 12]
+    for prompt, tokens in zip(res["prompts"], res["generated"]):
+        ids = list(prompt)
+        for k, tok in enumerate(tokens):
+            row = P.forward(w, cfg, ids)[-1]
+            twin = int(row.argmax())
+            if twin != tok:
+                margin = float((row[twin] - row[tok]) / row.abs().max())
+                assert margin < TOL["float32"], f"token {k} is {tok}, plainly {twin} (margin {margin:.2e})"
+            ids.append(tok)
+
+
+@pytest.mark.parametrize("dtype,extra", [("float32", ("--page-size", "8", "--poison")), ("bfloat16", ("--graphs",))])
+def test_trace_run_as_a_process(dtype, extra, folders, tmp_path):
+    from test_trace_run_gpu import run_trace
+
+    folder, cfg, w = folders["small" if dtype == "float32" else "small16"]
+    vocab = cfg["vocab"]
+    reqs = {"a": random_ids(vocab, 70, 1), "b": random_ids(vocab, 40, 2), "c": random_ids(vocab, 64, 3), "d": random_ids(vocab, 3, 4),
+            "e": random_ids(vocab, 61, 5)}
+    fed = {r: 0 for r in reqs}
+    sizes = [13, 2, 30, 1, 7, 64, 3]
+    live, waiting, steps, k, wanted = [], list(reqs), [], 0, {}
+    while live or waiting:
+        while waiting and len(live) < 4:
+            live.append(waiting.pop(0))
+        entries, end = [], []
+        for r in live:
+            n = min(sizes[k % len(sizes)], len(reqs[r]) - fed[r])
+            k += 1
+            want = [] if k % 5 == 0 else list(range(0, n, 2))
+            entries.append({"id": r, "tokens": reqs[r][fed[r]:fed[r] + n], "want": want})
+            wanted.setdefault(len(steps), []).extend((r, fed[r] + x) for x in want)
+            fed[r] += n
+            if fed[r] == len(reqs[r]):
+                end.append(r)
+        steps.append({"step": len(steps), "entries": entries, "end": end})
+        live = [r for r in live if r not in end]
+    out = tmp_path / "out"
+    run_trace(folder, dtype, out, 4 * 128, steps, extra)
+    ref = {r: plain_rows(cfg, w, ids) for r, ids in reqs.items()}
+    calls = {r: P.closest_call(w, cfg, ids) for r, ids in reqs.items()}
+    checked = 0
+    for st, rows in wanted.items():
+        if not rows:
+            assert not (out / f"{st}.f32").exists()
+            continue
+        got = torch.from_numpy(np.fromfile(out / f"{st}.f32", dtype="<f4").reshape(len(rows), vocab))
+        for i, (r, pos) in enumerate(rows):
+            if dtype == "bfloat16" and (pos == 0 or float(calls[r][pos]) < CLOSE_CALL):
+                continue  # see assert_close
+            d = float((got[i] - ref[r][pos]).abs().max() / ref[r][pos].abs().max())
+            assert d <= TOL[dtype], f"step {st} request {r} position {pos}: {d:.3e}"
+            checked += 1
+    assert checked > 50
