@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--model qwen2.5-7b]
     python bench.py --workload serve [--model qwen2.5-1.5b] [--requests 256] [--max-batch 256]
-    python bench.py --workload designs [--shapes 1.5b,7b] [--layers 4] [--designs qwen2,mafurax,nurasun,durelix]
+    python bench.py --workload designs [--shapes 1.5b,7b] [--layers 4] [--designs qwen2,mafurax,nurasun,durelix,zorulix]
 
 A step is one decode step of the scheduler: every running request gets one new
 token (plan, one engine step over the paged cache, greedy sampling, token fed
@@ -38,7 +38,10 @@ elements, every second such layer reading the rows of the one before), and betwe
 same width and a mixture of 8 experts of a quarter of that width, of which a token takes 2 beside a
 shared expert of half the width (so a token's feed-forward work is the dense one's), and the Durelix design at
 the Mafurax design's split of the heads (a window of 1,024 tokens behind a convolution of four taps; layers alternate
-between down(relu(up)^2) of the same width and a mixture of 8 gated experts of a quarter of it and 4 identity experts).
+between down(relu(up)^2) of the same width and a mixture of 8 gated experts of a quarter of it and 4 identity experts),
+and the Zorulix design, whose layers alternate between attention over a window of 1,024 tokens (every second such layer
+reading the keys and values of the one before) and windowed attention beside the gated delta rule at the same split of
+the heads, every layer with the mixture of 8 gated experts and a shared one and with 64 columns of a second token table.
 For each:
 the prefill of a 2,048-token prompt, decode steps at 8 and 64 requests with contexts of 4,096, and
 the device time of every kernel of a prefill step and of a decode step at 8 requests.
@@ -267,7 +270,29 @@ def designs(args) -> dict:
                    "embedding": {"bigram": {"buckets": 65521, "mul_prev": 1000003, "mul_cur": 31}},
                    "layers": [{"type": "parallel", "mixer": {"left": dleft, "right": dright},
                                "mlp": dmix if i % 2 else {"kind": "dense", "ff": sh["ff"]}} for i in range(layers)]}
-        made = {"qwen2": qwen, "mafurax": mafurax, "nurasun": nurasun, "durelix": durelix}
+        # Zorulix: layers alternate between attention over a window of 1,024 tokens (all heads, half of each turned; every
+        # second such layer reading the keys and values of the one before) and the two branches side by side at the
+        # Mafurax design's split of the heads (the same window with stretched frequencies; the gated delta rule behind a
+        # convolution of four taps); every layer has the Nurasun design's mixture (8 gated experts of a quarter of the
+        # width, 2 taken, beside a shared expert of half of it) and takes 64 columns of the second token table
+        zatt = {"heads": sh["heads"], "kv_heads": sh["kv_heads"], "dim": sh["head"], "vdim": sh["head"], "scale": sh["head"] ** -0.5,
+                "mask": {"size": 1024}, "rot": {"base": 1e6, "dims": sh["head"] // 2}}
+        zleft = {"heads": sh["heads"] // 2, "kv_heads": max(1, sh["kv_heads"] // 2), "dim": sh["head"], "vdim": sh["head"],
+                 "scale": sh["head"] ** -0.5, "mask": {"size": 1024},
+                 "rot": {"base": 1e4, "dims": sh["head"], "scaling": {"factor": 4.0, "original": 1024, "fast": 32.0, "slow": 1.0}}}
+        zright = {"heads": sh["heads"] // 2, "kv_heads": sh["heads"] // 2, "dim": sh["head"], "vdim": sh["head"], "conv": 4}
+        zmix = {"kind": "moe", "router": {"experts": 8, "top": 2}, "expert": {"ff": sh["ff"] // 4}, "shared": {"ff": sh["ff"] // 2}}
+        zlayers, owner = [], None
+        for i in range(layers):
+            if i % 2:
+                zlayers.append({"type": "parallel", "mlp": zmix,
+                                "mixer": {"left": zleft, "right": zright, "left_scale": 1.0, "right_scale": 1.0}})
+            else:
+                zlayers.append({"type": "attention", "mlp": zmix, "mixer": dict(zatt, kv_from=owner) if owner is not None else zatt})
+                owner = i if owner is None else None
+        zorulix = {"architecture": "Zorulix", "vocab": sh["vocab"], "width": sh["width"], "norm": {"eps": 1e-6},
+                   "embedding": {"scale": 1.0}, "token_side": {"dim": 64}, "layers": zlayers}
+        made = {"qwen2": qwen, "mafurax": mafurax, "nurasun": nurasun, "durelix": durelix, "zorulix": zorulix}
         return {name: config_from_dict(made[name]) for name in args.designs.split(",") if name}
 
     def kernels_of(run, per: int) -> dict:
@@ -416,8 +441,8 @@ def main() -> int:
     ap.add_argument("--model", default=None, help="preset shape (qwen2.5-7b; for --workload serve qwen2.5-1.5b)")
     ap.add_argument("--workload", default="decode", choices=["decode", "serve", "designs"])
     ap.add_argument("--shapes", default="1.5b,7b", help="designs: the layer sizes to compare at (1.5b, 7b)")
-    ap.add_argument("--designs", default="qwen2,mafurax,nurasun,durelix",
-                    help="designs: which of qwen2, mafurax, nurasun, durelix to measure")
+    ap.add_argument("--designs", default="qwen2,mafurax,nurasun,durelix,zorulix",
+                    help="designs: which of qwen2, mafurax, nurasun, durelix, zorulix to measure")
     ap.add_argument("--requests", type=int, default=256, help="serve: number of requests")
     ap.add_argument("--max-batch", type=int, default=256, help="serve: requests that run at a time")
     ap.add_argument("--seed", type=int, default=0, help="serve: seed of the lengths and token ids")

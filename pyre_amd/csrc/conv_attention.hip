@@ -100,29 +100,6 @@ __global__ __launch_bounds__(kThreads) void conv_qkv_write_kernel(
 // 0 .. nq + nkv - 1 of a token take a head each, the blocks behind them 256 value or gate columns each. Head sizes, the
 // product's width, first column and stride are multiples of four; queries and caches share one element type. The sums
 // run in the order of the kernel above: the same bits.
-constexpr int kVecTaps = 8;  // the most taps of this form
-template <typename TP>
-__device__ inline float4 conv_value4(const ConvIn& in, const TP* proj, int n, int run, int slot, int ch) {
-  const TP* row = proj + static_cast<size_t>(n) * in.ld + in.col0 + ch;
-  if (!in.taps_w) return sum_partials4(row, in.partial_stride, in.n_partials);
-  float4 u[kVecTaps];
-#pragma unroll
-  for (int j = 0; j < kVecTaps; ++j) {  // every tap's input asked for before the first is used
-    if (j >= in.taps) break;
-    const int back = in.taps - 1 - j;
-    if (run - back >= 0) u[j] = sum_partials4(row - static_cast<size_t>(back) * in.ld, in.partial_stride, in.n_partials);
-    else u[j] = *reinterpret_cast<const float4*>(in.state + (static_cast<size_t>(slot) * (in.taps - 1) + (in.taps - 1 + run - back)) * in.channels + ch);
-  }
-  float4 y = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int j = 0; j < kVecTaps; ++j) {
-    if (j >= in.taps) break;
-    const float4 w = *reinterpret_cast<const float4*>(in.taps_w + static_cast<size_t>(j) * in.channels + ch);
-    y = float4{fmaf(w.x, u[j].x, y.x), fmaf(w.y, u[j].y, y.y), fmaf(w.z, u[j].z, y.z), fmaf(w.w, u[j].w, y.w)};
-  }
-  return y;
-}
-
 template <typename TP, typename TC>
 __global__ __launch_bounds__(kWave) void conv_qkv_write_vec_kernel(
     ConvIn in, const int* __restrict__ state_slots, const int* __restrict__ seq_of_token, const int* __restrict__ q_start,
@@ -213,7 +190,7 @@ extern "C" int pyre_conv_qkv_write(const void* proj, int proj_dt, int n_partials
                   (nq + nkv) * dk + nkv * dv};
   const auto a16 = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
   const int tail_blocks = (nkv * dv + (gate_out ? nq * dv : 0) + 4 * kWave - 1) / (4 * kWave);
-  if (taps <= kVecTaps && dk % 4 == 0 && dv % 4 == 0 && ld % 4 == 0 && col0 % 4 == 0 && partial_stride % 4 == 0 && q_dt == cache_dt &&
+  if (taps <= kConvVecTaps && dk % 4 == 0 && dv % 4 == 0 && ld % 4 == 0 && col0 % 4 == 0 && partial_stride % 4 == 0 && q_dt == cache_dt &&
       nq + nkv + tail_blocks <= 65535 && a16(proj) && a16(q_out) && a16(k_cache) && a16(v_cache) && a16(gate_out) &&
       a16(taps_w) && a16(conv_state) && a16(q_gain) && a16(k_gain)) {
     PYRE_DISPATCH(proj_dt, TP, PYRE_DISPATCH(cache_dt, TC,

@@ -129,8 +129,10 @@ extern "C" int pyre_add_rmsnorm(float* resid, const void* delta, int delta_dt, i
   PYRE_REQUIRE(!bias || known_dtype(bias_dt), "add_rmsnorm: unknown bias dtype");
   PYRE_REQUIRE(n >= 0 && hidden > 0 && eps > 0.f, "add_rmsnorm: bad sizes n=%d hidden=%d", n, hidden);
   if (n == 0) return 0;
-  if (!bias && add_rmsnorm_vec(resid, delta, delta_dt, delta ? n_partials : 0, partial_stride, gain, gain_dt,
-                               out, out_dt, rows, n, hidden, eps, stream))
+  // (a pending bias of float32 rides along in the vectorised form; one of another type takes the general kernel)
+  if ((!bias || bias_dt == kF32) &&
+      add_rmsnorm_vec(resid, delta, delta_dt, delta ? n_partials : 0, partial_stride, static_cast<const float*>(bias), gain,
+                      gain_dt, out, out_dt, rows, n, hidden, eps, stream))
     return check_launch("add_rmsnorm");
   hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(n), dim3(256), 0, stream, resid, delta, delta_dt,
                      n_partials, static_cast<size_t>(partial_stride), bias, bias_dt, gain, gain_dt,

@@ -54,7 +54,8 @@ constexpr int kNormMaxVec = 8;  // float4 per thread
 template <typename TD, typename TG, typename TO, int THREADS, int VIRT, bool STREAM>
 __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(
     float* __restrict__ resid, const TD* __restrict__ delta, int n_partials, size_t partial_stride,
-    const TG* __restrict__ gain, TO* __restrict__ out, const int* __restrict__ rows, int hidden, float eps) {
+    const float* __restrict__ bias, const TG* __restrict__ gain, TO* __restrict__ out, const int* __restrict__ rows, int hidden,
+    float eps) {
   __shared__ float scratch[16];
   const int r_out = blockIdx.x, r_in = rows ? rows[r_out] : r_out;
   const size_t in_off = static_cast<size_t>(r_in) * hidden;
@@ -76,6 +77,7 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(
       } else {
         d = sum_partials4<TD>(delta + in_off + 4 * c, partial_stride, n_partials);
       }
+      if (bias) d = add4(d, Vec4<float>::load(bias + 4 * c));  // all partial sums, then the bias
       x = add4(x, d);
       if (!rows) {
         if (STREAM) Stream4<float>::store(resid + in_off + 4 * c, x);
@@ -234,15 +236,16 @@ __global__ __launch_bounds__(256) void silu_mul_stream_kernel(const bf16* __rest
 namespace pyre {
 
 bool add_rmsnorm_vec(float* resid, const void* delta, int delta_dt, int n_partials, long partial_stride,
-                     const void* gain, int gain_dt, void* out, int out_dt, const int* rows, int n,
+                     const float* bias, const void* gain, int gain_dt, void* out, int out_dt, const int* rows, int n,
                      int hidden, float eps, hipStream_t stream) {
   if (hidden % 4 || hidden > 4 * 256 * kNormMaxVec || (delta && partial_stride % 4)) return false;
+  if (bias && (!delta || reinterpret_cast<uintptr_t>(bias) % 16)) return false;
   // Which variant runs depends on the number of rows; what it computes does not (see the kernel).
   const bool wide = hidden > 1024;
   const bool few = n <= 128 && wide;  // a decode step: spread each row over more threads
 #define PYRE_NORM_LAUNCH(THREADS, VIRT, STREAM)                                                                      \
   hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TG, TO, THREADS, VIRT, STREAM>), dim3(n), dim3(THREADS), 0, stream, \
-                     resid, static_cast<const TD*>(delta), n_partials, static_cast<size_t>(partial_stride),          \
+                     resid, static_cast<const TD*>(delta), n_partials, static_cast<size_t>(partial_stride), bias,    \
                      static_cast<const TG*>(gain), static_cast<TO*>(out), rows, hidden, eps)
   PYRE_DISPATCH(delta_dt, TD, PYRE_DISPATCH(gain_dt, TG, PYRE_DISPATCH(out_dt, TO, {
     const bool many = n >= 512;  // more bytes than the caches keep for the next kernel

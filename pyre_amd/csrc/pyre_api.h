@@ -370,8 +370,9 @@ int pyre_gdr_prepare(const void* proj, int proj_dt, int n_partials, long partial
                      const int* seq_of_token, const int* q_start, int n_seqs, const void* a2, int a2_dt,
                      const float* dt_bias, const float* rate, const void* g2, int g2_dt, float unit_eps, float* x, int n,
                      int H, int G, int dk, int dv, int rank_a, int rank_g, hipStream_t stream);
-int pyre_gdr_scan(const float* x, float* state, float* o, const int* q_start, const int* state_slots, int n_seqs, int H,
-                  int G, int dk, int dv, hipStream_t stream);
+// state [slots][H][dv][dk]: a column's rows lie together; max_tokens: the most tokens that one request brings (0: unknown)
+int pyre_gdr_scan(const float* x, float* state, float* o, const int* q_start, const int* state_slots, int n_seqs,
+                  int max_tokens, int H, int G, int dk, int dv, hipStream_t stream);
 int pyre_gdr_finish(const float* o, const float* x, const void* gain, int gain_dt, float eps, float out_scale, void* out,
                     int out_dt, long out_ld, int n, int H, int G, int dk, int dv, hipStream_t stream);
 

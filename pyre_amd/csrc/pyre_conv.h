@@ -4,6 +4,7 @@
 #pragma once
 
 #include "pyre_common.h"
+#include "pyre_vec4.h"
 
 namespace pyre {
 
@@ -39,6 +40,35 @@ __device__ inline float conv_value(const ConvIn& in, int n, int run, int slot, i
     if (run - back >= 0) u = product_value(in, n - back, ch);
     else u = in.state[(static_cast<size_t>(slot) * (in.taps - 1) + (in.taps - 1 + run - back)) * in.channels + ch];
     y = fmaf(in.taps_w[static_cast<size_t>(j) * in.channels + ch], u, y);
+  }
+  return y;
+}
+
+// Four neighbouring channels at a time (the product's width, first column and stride, the channels and `ch` are multiples
+// of four, the pointers on 16 bytes): every tap's input asked for before the first is used; the same sums in the same
+// order as conv_value.
+constexpr int kConvVecTaps = 8;  // the most taps of this form
+template <typename TP>
+__device__ inline float4 conv_value4(const ConvIn& in, const TP* proj, int n, int run, int slot, int ch) {
+  const TP* row = proj + static_cast<size_t>(n) * in.ld + in.col0 + ch;
+  const float4 b = in.bias ? *reinterpret_cast<const float4*>(in.bias + in.col0 + ch) : float4{0.f, 0.f, 0.f, 0.f};
+  if (!in.taps_w) return in.bias ? add4(sum_partials4(row, in.partial_stride, in.n_partials), b) : sum_partials4(row, in.partial_stride, in.n_partials);
+  float4 u[kConvVecTaps];
+#pragma unroll
+  for (int j = 0; j < kConvVecTaps; ++j) {  // every tap's input asked for before the first is used
+    if (j >= in.taps) break;
+    const int back = in.taps - 1 - j;
+    if (run - back >= 0) {
+      u[j] = sum_partials4(row - static_cast<size_t>(back) * in.ld, in.partial_stride, in.n_partials);
+      if (in.bias) u[j] = add4(u[j], b);
+    } else u[j] = *reinterpret_cast<const float4*>(in.state + (static_cast<size_t>(slot) * (in.taps - 1) + (in.taps - 1 + run - back)) * in.channels + ch);
+  }
+  float4 y = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < kConvVecTaps; ++j) {
+    if (j >= in.taps) break;
+    const float4 w = *reinterpret_cast<const float4*>(in.taps_w + static_cast<size_t>(j) * in.channels + ch);
+    y = float4{fmaf(w.x, u[j].x, y.x), fmaf(w.y, u[j].y, y.y), fmaf(w.z, u[j].z, y.z), fmaf(w.w, u[j].w, y.w)};
   }
   return y;
 }

@@ -7,7 +7,7 @@
 namespace pyre {
 
 bool add_rmsnorm_vec(float* resid, const void* delta, int delta_dt, int n_partials, long partial_stride,
-                     const void* gain, int gain_dt, void* out, int out_dt, const int* rows, int n,
+                     const float* bias, const void* gain, int gain_dt, void* out, int out_dt, const int* rows, int n,
                      int hidden, float eps, hipStream_t stream);
 
 bool rope_kv_write_vec(const void* qkv, int qkv_dt, int n_partials, long partial_stride, const void* bias,

@@ -84,7 +84,7 @@ _SIGNATURES = {
     "pyre_add_weighted_rows": [P, P, I, L, P, L, I, I, I, I, P],
     "pyre_wide_norm_qkv_write": [P, I, I, L, I, I, P, P, P, F, P, P, I, P, P, I, P, P, I, P, I, I, I, I, I, I, I, P],
     "pyre_gdr_prepare": [P, I, I, L, I, I, P, P, I, P, P, P, P, I, P, I, P, P, P, I, F, P, I, I, I, I, I, I, I, P],
-    "pyre_gdr_scan": [P, P, P, P, P, I, I, I, I, I, P],
+    "pyre_gdr_scan": [P, P, P, P, P, I, I, I, I, I, I, P],
     "pyre_gdr_finish": [P, P, P, I, F, F, P, I, L, I, I, I, I, I, P],
     "pyre_token_side_gate": [P, I, I, L, P, I, P, I, I, I, P, P, I, I, I, P],
 }

@@ -1456,8 +1456,9 @@ GDR_MAX_RANK = 512   #: the widest low-rank input of its decay and of its gate
 
 
 def gdr_row_width(heads: int, kv_heads: int, dk: int, dv: int) -> int:
-    """Columns of the float32 rows [q | k | decay | v | gate | beta] that the gated delta rule's kernels share."""
-    return 2 * kv_heads * dk + heads * dk + 2 * heads * dv + heads
+    """Columns of the float32 rows [q | k | decay | v | gate | beta] that the gated delta rule's kernels share (rounded up
+    to a multiple of four, so that every row starts on 16 bytes)."""
+    return (2 * kv_heads * dk + heads * dk + 2 * heads * dv + heads + 3) // 4 * 4
 
 
 def gdr_prepare(proj: Partials, col0: int, taps_w: torch.Tensor | None, conv_state: torch.Tensor | None,
@@ -1499,19 +1500,21 @@ def gdr_prepare(proj: Partials, col0: int, taps_w: torch.Tensor | None, conv_sta
 
 
 def gdr_scan(x: torch.Tensor, state: torch.Tensor, o: torch.Tensor, q_start: torch.Tensor, state_slots: torch.Tensor,
-             n_seqs: int, heads: int, kv_heads: int, dk: int, dv: int) -> None:
-    """The gated delta rule over each request's tokens of the step, from and into ``state [slots, heads, dk, dv]``:
-    S <- diag(decay) S; u = beta (v - S^T k); S <- S + k u^T; ``o`` (float32 [N, heads*dv]) receives S^T q."""
+             n_seqs: int, heads: int, kv_heads: int, dk: int, dv: int, max_tokens: int = 0) -> None:
+    """The gated delta rule over each request's tokens of the step, from and into ``state [slots, heads, dv, dk]`` (the
+    state S [dk, dv] of a head kept column by column): S <- diag(decay) S; u = beta (v - S^T k); S <- S + k u^T; ``o``
+    (float32 [N, heads*dv]) receives S^T q. ``max_tokens``: the most tokens that one request brings (0: unknown); a step
+    of single tokens is launched with less shared memory a block."""
     _dev(x, state, o, q_start, state_slots)
     for name, t in (("x", x), ("state", state), ("o", o)):
         if t.dtype != torch.float32 or not t.is_contiguous():
             raise KernelError(f"gdr_scan: {name} is contiguous float32")
-    if tuple(state.shape[1:]) != (heads, dk, dv) or x.shape[-1] != gdr_row_width(heads, kv_heads, dk, dv) or \
+    if tuple(state.shape[1:]) != (heads, dv, dk) or x.shape[-1] != gdr_row_width(heads, kv_heads, dk, dv) or \
             o.shape[-1] != heads * dv:
         raise KernelError("gdr_scan: shapes do not fit the head geometry")
     _i32("q_start", q_start, n_seqs + 1), _i32("state_slots", state_slots, n_seqs)
     call("pyre_gdr_scan", x.data_ptr(), state.data_ptr(), o.data_ptr(), q_start.data_ptr(), state_slots.data_ptr(), n_seqs,
-         heads, kv_heads, dk, dv, _stream())
+         int(max_tokens), heads, kv_heads, dk, dv, _stream())
 
 
 def gdr_finish(o: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, eps: float, out_scale: float, out: torch.Tensor,

@@ -49,6 +49,9 @@ class PreNormBlock(Block):
     def bind(self, tensors, runtime) -> None:
         for p in self.parts():
             p.bind(tensors, runtime)
+        if self.token_input_norm is not None and self.mixer_norm.gain.dtype == torch.float32:
+            # the kernel that adds a normed term and norms the sum takes one element type for all its gains
+            self.token_input_norm.gain = self.token_input_norm.gain.float().contiguous()
 
     def linears(self) -> list:
         return [lin for p in self.parts() for lin in p.linears()]

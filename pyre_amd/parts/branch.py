@@ -67,6 +67,13 @@ class BranchMixer(Mixer):
     def bind(self, tensors, runtime) -> None:
         bias = _in_bias(self, tensors)
         w = _stacked([s.name for s in self.in_tensors()], tensors, 0)  # a size that only the file knows is known now
+        pad = -w.shape[0] % COLUMN_ALIGN
+        if pad:
+            # rows of zeros behind a product whose width is no multiple of eight: its rows then start on 16 bytes,
+            # which the kernels that finish it four columns at a time need
+            w = torch.cat([w, torch.zeros(pad, w.shape[1], dtype=w.dtype, device=w.device)], dim=0)
+            if bias is not None:
+                bias.append(torch.zeros(pad, dtype=torch.float32, device=w.device))
         self._in = Linear(self.hidden_size, w.shape[0], f"{self.role}.in")
         self._out = Linear(self.inner, self.hidden_size, f"{self.role}.out")
         self._in.set(w, None if bias is None else torch.cat(bias))
@@ -160,8 +167,8 @@ class ParallelMixer(Mixer):
             bias = _in_bias(b, tensors)
             mine = [take(tensors, s.name) for s in b.in_tensors()]
             rows = sum(t.shape[0] for t in mine)
-            pad = -rows % COLUMN_ALIGN
-            if pad and b is not self.branches[-1]:
+            pad = -rows % COLUMN_ALIGN   # (behind the last branch too: the product's rows then start on 16 bytes)
+            if pad:
                 mine.append(torch.zeros(pad, mine[0].shape[1], dtype=mine[0].dtype, device=mine[0].device))
                 rows += pad
             biases.append(bias if bias is None else torch.cat(bias + [torch.zeros(rows - sum(x.numel() for x in bias),

@@ -19,7 +19,7 @@ class GatedDeltaRule(BranchMixer):
     a = exp(-exp(A_log) softplus(A2 (A1 h) + dt_bias)) per key channel; o / rms(o) * gain * sigmoid(G2 (G1 h)); then the
     output matrix. All its input matrices (B, A1 and G1 among them) are one product.
 
-    Keeps two states per request: S [heads, key_dim, value_dim] float32 and the last ``taps - 1`` projected rows of q, k
+    Keeps two states per request: S float32 [heads, value_dim, key_dim] (column by column) and the last ``taps - 1`` projected rows of q, k
     and v, which the convolution of the next step's first tokens reads."""
 
     role = "gdr"
@@ -42,7 +42,8 @@ class GatedDeltaRule(BranchMixer):
 
     def cache_spec(self):
         s = self.spec
-        return StateCacheSpec((s.num_heads, s.key_dim, s.value_dim), "float32")
+        # a head's state S [key_dim, value_dim] column by column: the rows of a column lie together for the kernel
+        return StateCacheSpec((s.num_heads, s.value_dim, s.key_dim), "float32")
 
     def cache_specs(self) -> list:
         specs = [self.cache_spec()]
@@ -97,5 +98,5 @@ class GatedDeltaRule(BranchMixer):
         ops.gdr_prepare(proj, col0, self.taps, conv.tensor if conv is not None else None, ctx.state_slots,
                         ctx.seq_of_token, ctx.q_start, ctx.n_seqs, self.a2, self.dt_bias, self.rate, self.g2, s.unit_eps,
                         x, n, *shape)
-        ops.gdr_scan(x, state.tensor, raw, ctx.q_start, state.slots, ctx.n_seqs, *shape)
+        ops.gdr_scan(x, state.tensor, raw, ctx.q_start, state.slots, ctx.n_seqs, *shape, max_tokens=ctx.host.max_q_len)
         ops.gdr_finish(raw, x, self.gain, s.norm_eps, scale, o, n, *shape)

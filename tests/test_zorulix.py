@@ -62,7 +62,7 @@ def test_configuration_round_trip_and_manifest(raw):
             assert names[f"{p}.mix.right.a1"] == (None, width) and names[f"{p}.mix.right.o"] == (width, r["heads"] * r["vdim"])
             channels = 2 * r["kv_heads"] * r["dim"] + r["heads"] * r["vdim"]
             states = [s.shape for s in kept[i] if isinstance(s, StateCacheSpec)]
-            assert states == [(r["heads"], r["dim"], r["vdim"])] + ([(r["conv"] - 1, channels)] if r["conv"] > 1 else [])
+            assert states == [(r["heads"], r["vdim"], r["dim"])] + ([(r["conv"] - 1, channels)] if r["conv"] > 1 else [])
             assert [s.window for s in kept[i] if isinstance(s, PagedCacheSpec)] == [(a.get("mask") or {}).get("size", 0)]
         mlp = layer["mlp"]
         assert (f"{p}.norm2" in names) == (mlp is not None)

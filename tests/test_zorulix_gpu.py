@@ -480,7 +480,8 @@ def test_the_kernel_that_norms_a_whole_projection(nq, nkv, dk, dv, rot):
                 assert float((vt - vw).abs().max()) < tol * float(vw.abs().max())
 
 
-@pytest.mark.parametrize("H,G,dk,dv", [(2, 1, 8, 8), (3, 3, 33, 70), (4, 2, 130, 5), (1, 1, 1, 1)])
+@pytest.mark.parametrize("H,G,dk,dv", [(2, 1, 8, 8), (3, 3, 33, 70), (4, 2, 130, 5), (1, 1, 1, 1), (2, 1, 16, 24), (4, 2, 128, 130),
+                                       (3, 3, 48, 16), (1, 1, 112, 7)])
 def test_the_delta_rule_kernels(H, G, dk, dv):
     """The recurrence alone, from a state that is not empty, over requests of unequal lengths in one launch; then its
     finishing kernel."""
@@ -492,7 +493,7 @@ def test_the_delta_rule_kernels(H, G, dk, dv):
     x = torch.randn(n, width, generator=g)
     a0, v0, g0, b0 = 2 * G * dk, 2 * G * dk + H * dk, 2 * G * dk + H * dk + H * dv, 2 * G * dk + H * dk + 2 * H * dv
     x[:, a0:v0] = torch.rand(n, H * dk, generator=g) * 0.5 + 0.5            # decays
-    x[:, b0:] = torch.rand(n, H, generator=g)                               # betas
+    x[:, b0:b0 + H] = torch.rand(n, H, generator=g)                         # betas
     x[:, g0:b0] = torch.rand(n, H * dv, generator=g)                        # gates
     state = torch.randn(5, H, dk, dv, generator=g)
     slots = [3, 0, 4]
@@ -510,13 +511,13 @@ def test_the_delta_rule_kernels(H, G, dk, dv):
                 want_state[s, hd] = S
                 want_o[t, hd] = S.T @ q
         t0 += ln
-    st, o = state.to(DEV), torch.empty(n, H * dv, device=DEV)
+    st, o = state.transpose(2, 3).contiguous().to(DEV), torch.empty(n, H * dv, device=DEV)  # kept column by column
     q_start = torch.tensor([0, 7, 8, 20], dtype=torch.int32, device=DEV)
     ops.gdr_scan(x.to(DEV), st, o, q_start, torch.tensor(slots, dtype=torch.int32, device=DEV), 3, H, G, dk, dv)
     scale = float(want_o.abs().max())
     assert float((o.cpu().double().reshape(n, H, dv) - want_o).abs().max()) < 2e-5 * scale
-    assert float((st.cpu().double() - want_state).abs().max()) < 2e-5 * float(want_state.abs().max())
-    assert torch.equal(st[[1, 2]].cpu(), state[[1, 2]])
+    assert float((st.cpu().double().transpose(2, 3) - want_state).abs().max()) < 2e-5 * float(want_state.abs().max())
+    assert torch.equal(st[[1, 2]].cpu().transpose(2, 3), state[[1, 2]])
     gain = 1 + 0.2 * torch.randn(dv, generator=g)
     want = P.unit_rms(want_o, 1e-4) * gain.double() * x[:, g0:b0].double().reshape(n, H, dv) * 0.7
     for dtype, tol in ((torch.float32, 3e-5), (torch.bfloat16, 1e-2)):
