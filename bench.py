@@ -279,7 +279,7 @@ def designs(args) -> dict:
                 "mask": {"size": 1024}, "rot": {"base": 1e6, "dims": sh["head"] // 2}}
         zleft = {"heads": sh["heads"] // 2, "kv_heads": max(1, sh["kv_heads"] // 2), "dim": sh["head"], "vdim": sh["head"],
                  "scale": sh["head"] ** -0.5, "mask": {"size": 1024},
-                 "rot": {"base": 1e4, "dims": sh["head"], "scaling": {"factor": 4.0, "original": 1024, "fast": 32.0, "slow": 1.0}}}
+                 "rot": {"base": 1e4, "dims": sh["head"], "scaling": {"factor": 4.0, "original": 2048, "fast": 16.0, "slow": 2.0}}}
         zright = {"heads": sh["heads"] // 2, "kv_heads": sh["heads"] // 2, "dim": sh["head"], "vdim": sh["head"], "conv": 4}
         zmix = {"kind": "moe", "router": {"experts": 8, "top": 2}, "expert": {"ff": sh["ff"] // 4}, "shared": {"ff": sh["ff"] // 2}}
         zlayers, owner = [], None

@@ -288,7 +288,7 @@ __global__ __launch_bounds__(2 * kWave) void gdr_scan_lanes_kernel(const float* 
         if (from[j] >= 0 && t < t_end) in_flight[j] = *reinterpret_cast<const float4*>(x + static_cast<size_t>(t) * width + from[j]);
       }
       if (lane < kGroup && first + lane < t_end) beta = x[static_cast<size_t>(first + lane) * width + bo];
-      float* slot = ring[grp & 1];   // the walking wave left it at the barrier before this round
+      float* slot = ring[grp & 1];   // the walking wave left it at the barrier before this group
 #pragma unroll
       for (int j = 0; j < kMine; ++j)
         if (lane + kWave * j < kItems) *reinterpret_cast<float4*>(slot + to[j]) = in_flight[j];
