@@ -17,7 +17,7 @@ from pyre_amd.registry import config_from_dict
 F = torch.float64
 
 
-@pytest.mark.parametrize("raw", [M.SMALL, M.ONES, M.WIDE, M.ODD])
+@pytest.mark.parametrize("raw", [M.SMALL, M.ONES, M.WIDE, M.ODD, M.ORDER])
 def test_configuration_round_trip_and_manifest(raw):
     from pyre_amd.parts.base import PagedCacheSpec, StateCacheSpec
     from pyre_amd.parts.model import LayeredModel

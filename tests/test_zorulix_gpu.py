@@ -25,15 +25,16 @@ from pyre_amd.config.model import ModelConfig
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
-#: bounds on max |difference| / max |logit| of a position: float32 against the float64 plain run (the recurrent branch
-#: subtracts what the state already holds from a token's value and divides its output by its root mean square, which
-#: takes a float32 run of a hundred tokens to a few 1e-5 where the differences cancel); bfloat16 loosely (the float32
-#: runs are the exact ones; heads of ten elements and weights drawn at 0.2 make 16-bit rows noisy)
-TOL = {"float32": 5e-5, "bfloat16": 1e-1}
+#: bounds on max |difference| / max |logit| of a position: float32 against the float64 plain run. The recurrent branch
+#: subtracts what the state already holds from a token's value and divides its output by its root mean square; with
+#: weights drawn at 0.2 and heads of a few elements some positions are ill-conditioned (the plain implementation run in
+#: float32 is itself 5e-6 off there, ten times its median), and the engine's rows a few 1e-5. bfloat16 loosely (the
+#: float32 runs are the exact ones; heads of ten elements make 16-bit rows noisy)
+TOL = {"float32": 1e-4, "bfloat16": 1e-1}
 #: a 16-bit run is not compared where the plain router's choice hangs on less than this much of a logit (the logits are
 #: of the order of one, and a 16-bit run's are off by a few hundredths, now and then by a tenth and more)
 CLOSE_CALL = 0.25
-MODELS = {"small": (M.SMALL, 11), "ones": (M.ONES, 12), "wide": (M.WIDE, 13), "odd": (M.ODD, 14),
+MODELS = {"small": (M.SMALL, 11), "ones": (M.ONES, 12), "wide": (M.WIDE, 13), "odd": (M.ODD, 14), "order": (M.ORDER, 17),
           # for the 16-bit runs: one routed layer, the last, so that a close call spoils one position and not the rest
           "small16": (M.routed_last(M.SMALL), 15), "odd16": (M.routed_last(M.ODD), 16)}
 
@@ -111,7 +112,7 @@ def all_given_back(eng):
 # ----------------------------------------------------------------------------- whole prompts, layer by layer
 
 
-@pytest.mark.parametrize("name", ["small", "ones", "wide", "odd"])
+@pytest.mark.parametrize("name", ["small", "ones", "wide", "odd", "order"])
 def test_every_layer_of_a_whole_prompt(name, folders):
     from pyre_amd.engine.batch import Entry
 
@@ -130,7 +131,8 @@ def test_every_layer_of_a_whole_prompt(name, folders):
 
 # (the model of single heads of two and three elements runs in float32 only: in 16 bits its logits are mostly rounding)
 @pytest.mark.parametrize("name,dtype,page", [("small", "float32", 8), ("small16", "bfloat16", 16), ("ones", "float32", 4),
-                                             ("wide", "float32", 16), ("odd", "float32", 8), ("odd16", "bfloat16", 16)])
+                                             ("wide", "float32", 16), ("odd", "float32", 8), ("odd16", "bfloat16", 16),
+                                             ("order", "float32", 16)])
 def test_prefill_decode_and_portions_agree_with_plain(name, dtype, page, folders):
     folder, cfg, w = folders[name]
     reqs = {r: random_ids(cfg["vocab"], n, seed=n) for r, n in (("a", 90), ("b", 1), ("c", 37))}
@@ -149,7 +151,7 @@ def test_prefill_decode_and_portions_agree_with_plain(name, dtype, page, folders
 
 
 @pytest.mark.parametrize("name,dtype,poison", [("small", "float32", True), ("wide", "float32", True), ("small16", "bfloat16", False),
-                                               ("ones", "float32", True), ("odd", "float32", True)])
+                                               ("ones", "float32", True), ("odd", "float32", True), ("order", "float32", True)])
 def test_mixed_batches_with_pages_and_slots_used_again(name, dtype, poison, folders):
     folder, cfg, w = folders[name]
     reqs = {r: random_ids(cfg["vocab"], n, seed=7 * n) for r, n in (("a", 61), ("b", 9), ("c", 100), ("d", 33), ("e", 2), ("f", 47))}
@@ -377,7 +379,9 @@ def _build_one_mixer(cfg):
         p = f"l{i}.mix"
         if layer["type"] == "right":
             r = DeltaRuleConfig.from_dict(layer["mixer"], "right")
-            mixer = GatedDeltaRuleSpec(width, r.heads, r.kv_heads, r.dim, r.vdim, r.conv, p, norm_eps=eps)
+            ranks = layer.get("ranks") or (None, None)   # the two low-rank products need not agree in their rank
+            mixer = GatedDeltaRuleSpec(width, r.heads, r.kv_heads, r.dim, r.vdim, r.conv, p, norm_eps=eps, decay_rank=ranks[0],
+                                       gate_rank=ranks[1])
         else:
             a = AttentionConfig.from_dict(layer["mixer"], "left")
             whole = layer["type"] == "attention"
@@ -414,10 +418,14 @@ def test_each_mixer_alone(kind, tmp_path):
               "right": [M.delta(2, 2, 16, 24, 3), M.delta(6, 3, 33, 7, 1), M.delta(2, 1, 5, 70, 9)]}[kind]
     raw = {"architectures": ["ToyOneMixer"], "vocab": 71, "width": 40, "norm": {"eps": 1e-5},
            "layers": [{"type": kind, "mixer": m, "mlp": None} for m in mixers]}
+    if kind == "right":
+        raw["layers"][0]["ranks"], raw["layers"][2]["ranks"] = (5, 12), (16, 1)
     register_architecture(OneMixerConfig.architecture, OneMixerConfig, _build_one_mixer)
     try:
         write_random_model(tmp_path, OneMixerConfig(raw), seed=41, std=0.2, gain_std=0.2)
         _, w = P.read_folder(tmp_path)
+        if kind == "right":
+            assert w["l0.mix.a1"].shape[0] == 5 and w["l0.mix.g2"].shape[1] == 12 and w["l2.mix.a2"].shape[1] == 16
         reqs = {r: random_ids(71, n, seed=n) for r, n in (("a", 70), ("b", 19))}
         want = {r: _plain_one_mixer(w, raw, ids) for r, ids in reqs.items()}
         eng = engine_of(tmp_path, "float32")

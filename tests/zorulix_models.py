@@ -91,6 +91,18 @@ ODD = model(53, 50, [
 ], eps=1e-4)
 
 
+#: the recurrent layer first, one owner of keys read by two later layers through a narrower and a wider window than its
+#: own, with a parallel layer between them; rotation of part of a head everywhere; a key head of 16 and of 48 elements in
+#: the recurrent branches (the sizes that their kernel takes a wave a column group for)
+ORDER = model(80, 40, [
+    parallel(attn(2, 1, 24, 12, 0.3, window=14, rot=rot(2000.0, 10, (2.5, 20, 3.0, 0.7))), delta(4, 2, 16, 8, 2), 1.1, 0.6, moe(4, 2, 12, shared=6)),
+    attention(attn(6, 3, 10, 14, 0.35, window=16, rot=rot(700.0, 4)), moe(3, 1, 20)),
+    attention(attn(6, 3, 10, 14, 0.5, window=9, rot=rot(700.0, 4), kv_from=1), moe(8, 3, 6, shared=10)),
+    parallel(attn(3, 3, 8, 8, 0.45, rot=rot(90.0, 8)), delta(2, 2, 48, 20, 3), 0.9, 1.0),
+    attention(attn(6, 3, 10, 14, 0.2, window=26, rot=rot(700.0, 4), kv_from=1), moe(5, 5, 8, shared=4)),
+], eps=1e-5, scale=5.0, side=3)
+
+
 def routed_last(raw):
     """The same layers with a feed-forward in the last one only: a 16-bit run sends a token whose two experts nearly tie
     to another expert than the exact run does, a step and not a rounding, which in a last layer spoils that token's
