@@ -326,32 +326,39 @@ __global__ __launch_bounds__(2 * kWave) void gdr_scan_lanes_kernel(const float* 
       rv = tk[3 * kDk + lane / LPC];
       rb = tk[4 * kPieces];
     };
-    read(0, a, k, q, v, beta);
-    for (int i = 0; i < count; ++i) {
-      float4 an[DR / 4], kn[DR / 4], qn[DR / 4];
-      float vn, betan;
-      read(i + 1 < count ? i + 1 : i, an, kn, qn, vn, betan);   // the next token's rows come while this one is worked on
+    // one token: decay, the sum S^T k, the correction along k, the sum S^T q
+    auto step = [&](int i, const float4* ta, const float4* tk, const float4* tq, float tv, float tb) {
       float4 pk = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int r = 0; r < DR / 4; ++r) {
-        S[4 * r] *= a[r].x, S[4 * r + 1] *= a[r].y, S[4 * r + 2] *= a[r].z, S[4 * r + 3] *= a[r].w;
-        pk.x = fmaf(S[4 * r], k[r].x, pk.x), pk.y = fmaf(S[4 * r + 1], k[r].y, pk.y);
-        pk.z = fmaf(S[4 * r + 2], k[r].z, pk.z), pk.w = fmaf(S[4 * r + 3], k[r].w, pk.w);
+        S[4 * r] *= ta[r].x, S[4 * r + 1] *= ta[r].y, S[4 * r + 2] *= ta[r].z, S[4 * r + 3] *= ta[r].w;
+        pk.x = fmaf(S[4 * r], tk[r].x, pk.x), pk.y = fmaf(S[4 * r + 1], tk[r].y, pk.y);
+        pk.z = fmaf(S[4 * r + 2], tk[r].z, pk.z), pk.w = fmaf(S[4 * r + 3], tk[r].w, pk.w);
       }
-      const float u = beta * (v - lanes_sum<LPC>((pk.x + pk.y) + (pk.z + pk.w)));
+      const float u = tb * (tv - lanes_sum<LPC>((pk.x + pk.y) + (pk.z + pk.w)));
       float4 pq = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int r = 0; r < DR / 4; ++r) {
-        S[4 * r] = fmaf(k[r].x, u, S[4 * r]), S[4 * r + 1] = fmaf(k[r].y, u, S[4 * r + 1]);
-        S[4 * r + 2] = fmaf(k[r].z, u, S[4 * r + 2]), S[4 * r + 3] = fmaf(k[r].w, u, S[4 * r + 3]);
-        pq.x = fmaf(S[4 * r], q[r].x, pq.x), pq.y = fmaf(S[4 * r + 1], q[r].y, pq.y);
-        pq.z = fmaf(S[4 * r + 2], q[r].z, pq.z), pq.w = fmaf(S[4 * r + 3], q[r].w, pq.w);
+        S[4 * r] = fmaf(tk[r].x, u, S[4 * r]), S[4 * r + 1] = fmaf(tk[r].y, u, S[4 * r + 1]);
+        S[4 * r + 2] = fmaf(tk[r].z, u, S[4 * r + 2]), S[4 * r + 3] = fmaf(tk[r].w, u, S[4 * r + 3]);
+        pq.x = fmaf(S[4 * r], tq[r].x, pq.x), pq.y = fmaf(S[4 * r + 1], tq[r].y, pq.y);
+        pq.z = fmaf(S[4 * r + 2], tq[r].z, pq.z), pq.w = fmaf(S[4 * r + 3], tq[r].w, pq.w);
       }
       const float out = lanes_sum<LPC>((pq.x + pq.y) + (pq.z + pq.w));
       if (part == 0 && has_col) o[static_cast<size_t>(first + i) * s.H * s.dv + hd * s.dv + col] = out;
-#pragma unroll
-      for (int r = 0; r < DR / 4; ++r) a[r] = an[r], k[r] = kn[r], q[r] = qn[r];
-      v = vn, beta = betan;
+    };
+    // two sets of registers take turns: a token's rows are read while the token before it is worked on, and nothing
+    // is moved from one set to the other
+    float4 a2[DR / 4], k2[DR / 4], q2[DR / 4];
+    float v2, beta2;
+    read(0, a, k, q, v, beta);
+    for (int i = 0; i < count; i += 2) {
+      read(i + 1 < count ? i + 1 : i, a2, k2, q2, v2, beta2);
+      step(i, a, k, q, v, beta);
+      if (i + 1 < count) {
+        read(i + 2 < count ? i + 2 : i + 1, a, k, q, v, beta);
+        step(i + 1, a2, k2, q2, v2, beta2);
+      }
     }
     lds_barrier();   // done with this slot; the one after it is full
   }
